@@ -1,0 +1,137 @@
+/*
+ * C ABI of libcce_hip.so: Cut Cross-Entropy kernels for AMD gfx950 (MI355X).
+ *
+ * Every entry point is stream-ordered (work is enqueued on `stream`, a
+ * hipStream_t passed as void*), takes plain device pointers and sizes, never
+ * allocates device memory, never synchronises, and returns 0 on success or a
+ * non-zero status (a hipError_t value, or one of the CCE_ERR_* codes below).
+ * All scratch memory comes in through the `workspace` argument, sized by the
+ * matching *_workspace_bytes() query, so that a caller's allocator sees every
+ * byte the loss path uses.
+ *
+ * Each function names the reference interface it replaces
+ * (paths relative to the apple/ml-cross-entropy checkout).
+ *
+ * Common conventions
+ *   e        [n_rows, d]  row-major, row stride `stride_e` elements, unit column stride
+ *   c        [v, d]       row stride `stride_cv`, column stride `stride_cd` (elements)
+ *   valids   [b] int32    rows of `e` that take part (NULL: rows 0..b-1, b == n_rows)
+ *   targets  [n_rows] int64, read at (row + shift); a target t enters as
+ *            t - target_offset and matches no column when outside [0, v)
+ *   dtype    element type of e, c, bias: CCE_DTYPE_BF16 or CCE_DTYPE_F16
+ *   softcap  <= 0 (or NaN) switches soft-capping off
+ */
+#ifndef CCE_HIP_H
+#define CCE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CCE_OK 0
+#define CCE_ERR_INVALID_ARGUMENT 10001
+#define CCE_ERR_UNSUPPORTED_DTYPE 10002
+#define CCE_ERR_WORKSPACE_TOO_SMALL 10003
+#define CCE_ERR_MISALIGNED 10004
+
+#define CCE_DTYPE_BF16 0
+#define CCE_DTYPE_F16 1
+
+/* Granularity of the forward tile statistic (rows x vocabulary entries per cell). */
+#define CCE_STAT_ROWS 32
+#define CCE_STAT_COLS 128
+
+/* Number of uint64 slots in the backward counter block:
+ * [0] tiles in the grid, [1] tiles whose logits were recomputed,
+ * [2] tiles that ran the dE product, [3] tiles that ran the dC product. */
+#define CCE_NUM_COUNTERS 4
+
+/* Library ABI version (bumped when a signature below changes). */
+int cce_version(void);
+
+/* Human-readable text for a status returned by any function below. */
+const char* cce_error_string(int status);
+
+/* Number of floats in the forward tile statistic for b valid rows and v classes:
+ * ceil(b / CCE_STAT_ROWS) * ceil(v / CCE_STAT_COLS). */
+int64_t cce_tile_stat_elems(int64_t b, int64_t v);
+
+/* Scratch bytes cce_lse_forward needs (split-vocabulary partial max / sum-exp). */
+int64_t cce_lse_forward_workspace_bytes(int64_t b, int64_t v, int64_t d);
+
+/*
+ * lse[i] = log sum_v exp(softcap(e[valids[i]] . c[v] + bias[v])),  i in [0, b).
+ * Replaces cce_lse_forward_kernel (cut_cross_entropy/cce_lse_forward.py:170-237)
+ * and its Triton body (:12-117).
+ *   lse        [b] float, written (not accumulated)
+ *   logit_avg  NULL, or [v] float: receives (1/b) sum_i logit[i, v]  (reference :95-97)
+ *   tile_max   NULL, or [cce_tile_stat_elems(b, v)] float: max soft-capped logit of
+ *              every CCE_STAT_ROWS x CCE_STAT_COLS cell (row-major over cells); lets
+ *              cce_backward prove a tile filtered without recomputing it
+ */
+int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_t* valids,
+                    float* lse, float* logit_avg, float* tile_max,
+                    void* workspace, int64_t workspace_bytes,
+                    int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                    int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                    float softcap, int dtype, void* stream);
+
+/*
+ * out[i] = softcap(-(e[valids[i]] . c[t_i]) - bias[t_i]),  t_i = targets[valids[i] + shift] - target_offset;
+ * out[i] = 0 when t_i is outside [0, v).
+ * Replaces indexed_neg_dot_forward_kernel (cut_cross_entropy/indexed_dot.py:101-158,
+ * Triton body :11-85) including the soft-capping the reference applies on the host (:150-151).
+ */
+int cce_indexed_neg_dot(const void* e, const void* c, const int64_t* targets, const void* bias,
+                        const int32_t* valids, float* out,
+                        int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                        int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                        int64_t shift, int64_t target_offset,
+                        float softcap, int dtype, void* stream);
+
+/* Scratch bytes cce_backward needs (kept-tile list and its cursor). */
+int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d);
+
+/*
+ * Gradients of  sum_i d_out_i * nll_i + d_lse_i * lse_i  w.r.t. e, c and bias.
+ * Replaces cce_backward_kernel (cut_cross_entropy/cce_backward.py:346-521, Triton
+ * body :20-310).  Per valid row i and class v, with z the raw logit, s = softcap(z),
+ * p = exp(s - lse_i), y = [v == t_i], g = grad_scale * d_out_i, h = d_lse_i:
+ *     dz = (p (g + h) - y g) (1 - (s / softcap)^2)
+ *     d_e[row_i] += sum_v dz c[v];  d_c[v] += sum_i dz e[row_i];  d_bias[v] += sum_i dz.
+ * A tile of the (row, class) plane whose every |p - y| is below filter_eps is dropped
+ * from d_e when filter_e, from d_c when filter_c, and from d_bias when both are set
+ * (gradient filtering, reference :211-216).  filter_eps < 0 switches filtering off.
+ *
+ *   lse        [b] float      (the global LSE when c is a vocabulary shard)
+ *   d_out      [n_rows] float read at (row + shift), or one float when d_out_is_scalar
+ *   d_lse      NULL or [n_rows] float read at (row + shift)
+ *   vocab_order NULL or [v] int32 permutation of the classes; tiles are formed over the
+ *              permuted order (reference :153-155).  Disables the tile_max shortcut.
+ *   tile_max   NULL or the statistic written by cce_lse_forward for the same inputs
+ *   d_e        NULL or [n_rows, d] accumulated into (caller zero-fills); float when
+ *              d_e_is_fp32 else `dtype`; same strides as e
+ *   d_c        NULL or [v, d]; float when d_c_is_fp32 else `dtype`; same strides as c
+ *   d_bias     NULL or [v] float, accumulated into
+ *   counters   NULL or CCE_NUM_COUNTERS uint64, accumulated into
+ */
+int cce_backward(const void* e, const void* c, const void* bias,
+                 const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                 const int32_t* valids, const int32_t* vocab_order, const int64_t* targets,
+                 const float* tile_max,
+                 void* d_e, void* d_c, float* d_bias,
+                 void* workspace, int64_t workspace_bytes, uint64_t* counters,
+                 int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                 int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                 float grad_scale, float filter_eps, int filter_e, int filter_c,
+                 int d_e_is_fp32, int d_c_is_fp32,
+                 int64_t shift, int64_t target_offset,
+                 float softcap, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CCE_HIP_H */

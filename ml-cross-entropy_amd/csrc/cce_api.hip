@@ -1,0 +1,15 @@
+// Version and status text of the C ABI.
+#include "cce_common.h"
+
+extern "C" int cce_version(void) { return 1; }
+
+extern "C" const char* cce_error_string(int status) {
+  switch (status) {
+    case CCE_OK: return "success";
+    case CCE_ERR_INVALID_ARGUMENT: return "cce: invalid argument";
+    case CCE_ERR_UNSUPPORTED_DTYPE: return "cce: unsupported element type (bf16 and fp16 only)";
+    case CCE_ERR_WORKSPACE_TOO_SMALL: return "cce: workspace missing or too small";
+    case CCE_ERR_MISALIGNED: return "cce: pointer not aligned as required";
+    default: return hipGetErrorString(static_cast<hipError_t>(status));
+  }
+}

@@ -1,0 +1,272 @@
+// Shared device code of the gfx950 Cut Cross-Entropy kernels: element types, MFMA wrappers,
+// the global -> LDS tile loader and the LDS -> MFMA logit-tile main loop.
+//
+// Orientation used everywhere: the MFMA "A" operand is a tile of the classifier C (vocabulary
+// rows), the "B" operand a tile of the embeddings E (token rows), so a 32x32 accumulator block
+// holds logits^T: lane l owns token (l % 32) and the 16 vocabulary rows
+//     8 * (r / 4) + 4 * (l / 32) + (r % 4),  r = 0..15.
+// A lane therefore sees many classes of ONE token, which makes the per-token soft-max
+// statistics a register-local reduction.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cce_hip.h"
+
+namespace cce {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kBK = 64;          // reduction elements per LDS stage
+constexpr int kRowBytes = 128;   // kBK * sizeof(16-bit element)
+
+struct BF16 {};
+struct F16 {};
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<BF16> {
+  using vec8 = bf16x8_t;
+  static __device__ __forceinline__ float to_float(uint16_t bits) {
+    return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    __bf16 h = static_cast<__bf16>(f);
+    return __builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
+    bf16x2_t v;
+    v[0] = static_cast<__bf16>(lo);
+    v[1] = static_cast<__bf16>(hi);
+    __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<bf16x2_t*>(addr), v);
+  }
+};
+
+template <>
+struct Elem<F16> {
+  using vec8 = f16x8_t;
+  static __device__ __forceinline__ float to_float(uint16_t bits) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, bits));
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    _Float16 h = static_cast<_Float16>(f);
+    return __builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
+    f16x2_t v;
+    v[0] = static_cast<_Float16>(lo);
+    v[1] = static_cast<_Float16>(hi);
+    __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<f16x2_t*>(addr), v);
+  }
+};
+
+// Add `val` to one 16-bit float in global memory through a compare-and-swap on the aligned
+// 32-bit word that contains it (used where a packed two-element atomic would be misaligned).
+template <typename T>
+__device__ __forceinline__ void atomic_add_16(uint16_t* addr, float val) {
+  uintptr_t a = reinterpret_cast<uintptr_t>(addr);
+  unsigned int* word = reinterpret_cast<unsigned int*>(a & ~static_cast<uintptr_t>(3));
+  const bool high = (a & 2) != 0;
+  unsigned int old = *word, assumed;
+  do {
+    assumed = old;
+    uint16_t cur = high ? static_cast<uint16_t>(assumed >> 16) : static_cast<uint16_t>(assumed & 0xffffu);
+    uint16_t upd = Elem<T>::from_float(Elem<T>::to_float(cur) + val);
+    unsigned int next = high ? ((assumed & 0x0000ffffu) | (static_cast<unsigned int>(upd) << 16))
+                             : ((assumed & 0xffff0000u) | upd);
+    old = atomicCAS(word, assumed, next);
+  } while (old != assumed);
+}
+
+// Soft-capping in the log2 domain.  For a raw logit x returns s * log2(e) with
+// s = softcap * tanh(x / softcap) (or s = x when off) and the tanh value itself.
+struct Softcap {
+  float in_scale;   // 2 * log2(e) / softcap
+  float out_scale;  // softcap * log2(e)
+  int on;
+};
+
+__host__ __device__ inline Softcap make_softcap(float softcap) {
+  Softcap s;
+  s.on = (softcap > 0.0f) ? 1 : 0;  // false for NaN as well
+  s.in_scale = s.on ? 2.0f * kLog2e / softcap : 0.0f;
+  s.out_scale = s.on ? softcap * kLog2e : 0.0f;
+  return s;
+}
+
+// tanh(y) = 1 - 2 / (1 + exp(2 y)); exp2 overflow gives 1, underflow gives -1.
+__device__ __forceinline__ float softcap_log2(const Softcap& sc, float x, float& th) {
+  if (sc.on) {
+    float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
+    float w = __builtin_amdgcn_rcpf(1.0f + t);
+    th = 1.0f - 2.0f * w;
+    return sc.out_scale * th;
+  }
+  th = 0.0f;
+  return x * kLog2e;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = fminf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Global -> register -> LDS loader for ROWS rows of kBK 16-bit elements.
+// LDS image: row-major, 128 bytes per row, the eight 16-byte chunks of a row XOR-swizzled with
+// (row & 7) so that the 32 rows an MFMA operand fetch touches fall into distinct banks.
+// Thread t owns chunk (t & 7) of rows (t / 8) + q * (NT / 8).
+// ---------------------------------------------------------------------------------------------
+template <int ROWS, int NT, bool ALIGNED>
+struct RowLoader {
+  static constexpr int NQ = ROWS * 8 / NT;
+  static constexpr int ROWSTEP = NT / 8;
+  static_assert(ROWS * 8 % NT == 0, "tile rows must divide evenly over the threads");
+  static_assert(ROWSTEP % 8 == 0, "swizzle must not depend on q");
+
+  const uint16_t* ptr[NQ];  // row base or nullptr for a row outside the matrix
+  uint4 reg[NQ];
+
+  // ALIGNED: rows are 16-byte aligned, unit element stride and D % 8 == 0.
+  __device__ __forceinline__ void load(int k0, int D, int64_t stride_k) {
+    const int k = k0 + (threadIdx.x & 7) * 8;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (ALIGNED) {
+        if (ptr[q] != nullptr && k < D) v = *reinterpret_cast<const uint4*>(ptr[q] + k);
+      } else {
+        if (ptr[q] != nullptr) {
+          uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            uint32_t x = (k + i < D) ? static_cast<uint32_t>(ptr[q][static_cast<int64_t>(k + i) * stride_k]) : 0u;
+            w[i >> 1] |= x << ((i & 1) * 16);
+          }
+          v = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+      }
+      reg[q] = v;
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned char* lds) const {
+    const int row0 = threadIdx.x >> 3;
+    const int chunk = (threadIdx.x & 7) ^ (row0 & 7);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      *reinterpret_cast<uint4*>(lds + (row0 + q * ROWSTEP) * kRowBytes + (chunk << 4)) = reg[q];
+    }
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 lds_frag(const unsigned char* lds, int row, int chunk) {
+  uint4 v = *reinterpret_cast<const uint4*>(lds + row * kRowBytes + ((chunk ^ (row & 7)) << 4));
+  return __builtin_bit_cast(typename Elem<T>::vec8, v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// One logit tile: acc[vi][ti] += C_tile (TILE_V x D) * E_tile^T (D x TILE_T), both streamed through
+// two LDS stages of kBK columns.  Wave (wv, wt) of an NWV x NWT grid owns WV x WT accumulator
+// blocks of 32 x 32.  `lds` must hold 2 * (TILE_V + TILE_T) * 128 bytes.  Ends with a barrier, so
+// the LDS may be reused right after the call.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int WV, int WT, int NWV, int NWT, bool ALIGNED>
+struct LogitTile {
+  static constexpr int TILE_V = 32 * WV * NWV;
+  static constexpr int TILE_T = 32 * WT * NWT;
+  static constexpr int NT = 64 * NWV * NWT;
+  static constexpr int STAGE_BYTES = (TILE_V + TILE_T) * kRowBytes;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+
+  using CLoader = RowLoader<TILE_V, NT, ALIGNED>;
+  using ELoader = RowLoader<TILE_T, NT, ALIGNED>;
+
+  static __device__ __forceinline__ void run(f32x16 (&acc)[WV][WT], CLoader& cl, ELoader& el,
+                                             unsigned char* lds, int D, int64_t stride_ck) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wv = wave / NWT;
+    const int wt = wave % NWT;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[vi][ti][r] = 0.0f;
+
+    const int nk = (D + kBK - 1) / kBK;
+    cl.load(0, D, stride_ck);
+    el.load(0, D, 1);
+    cl.store(lds);
+    el.store(lds + TILE_V * kRowBytes);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+      unsigned char* cur = lds + (kt & 1) * STAGE_BYTES;
+      unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+      const bool more = (kt + 1) < nk;
+      if (more) {
+        cl.load((kt + 1) * kBK, D, stride_ck);
+        el.load((kt + 1) * kBK, D, 1);
+      }
+      const unsigned char* cbase = cur + (wv * WV * 32 + l32) * kRowBytes;
+      const unsigned char* ebase = cur + (TILE_V + wt * WT * 32 + l32) * kRowBytes;
+      const int sw = l32 & 7;
+#pragma unroll
+      for (int kk = 0; kk < kBK / 16; ++kk) {
+        typename Elem<T>::vec8 a[WV], b[WT];
+        const int coff = (((kk * 2 + half) ^ sw) << 4);
+#pragma unroll
+        for (int vi = 0; vi < WV; ++vi)
+          a[vi] = __builtin_bit_cast(typename Elem<T>::vec8,
+                                     *reinterpret_cast<const uint4*>(cbase + vi * 32 * kRowBytes + coff));
+#pragma unroll
+        for (int ti = 0; ti < WT; ++ti)
+          b[ti] = __builtin_bit_cast(typename Elem<T>::vec8,
+                                     *reinterpret_cast<const uint4*>(ebase + ti * 32 * kRowBytes + coff));
+#pragma unroll
+        for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+          for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(a[vi], b[ti], acc[vi][ti]);
+      }
+      if (more) {
+        cl.store(nxt);
+        el.store(nxt + TILE_V * kRowBytes);
+      }
+      __syncthreads();
+    }
+  }
+};
+
+inline int status_from_hip(hipError_t e) { return e == hipSuccess ? CCE_OK : static_cast<int>(e); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace cce

@@ -1,0 +1,329 @@
+// cce_lse_forward: fused (E . C^T) -> soft-cap -> online log-sum-exp for gfx950.
+//
+// Work decomposition.  The (row-block, vocabulary) plane is cut into items: one item is a block
+// of 256 valid rows times a contiguous span of 256-wide vocabulary tiles.  A workgroup (4 waves,
+// 2 x 2, each wave 128 classes x 128 rows of accumulators) owns one item, walks its span tile by
+// tile and keeps, per row, a running (max, sum-exp) pair in registers in the log2 domain.  At the
+// end the pairs of the two lane halves and of the two wave rows are merged and written as one
+// partial per (span, row); a second tiny kernel merges the spans.  No lock and no atomic is
+// needed and the result is deterministic.
+//
+// Workgroup ids are dealt round-robin to the 8 XCDs by the hardware, so the id is first turned
+// into (xcd, slot) and items are numbered so that one XCD works on neighbouring spans of the
+// same few row blocks: its L2 then serves each E block to several workgroups and each C tile to
+// several row blocks.
+#include "cce_common.h"
+
+namespace cce {
+
+struct LseFwdParams {
+  const uint16_t* e;
+  const uint16_t* c;
+  const uint16_t* bias;
+  const int32_t* valids;
+  float* logit_avg;
+  float* tile_max;
+  float2* partial;  // [nsplit][b] (max2, sum)
+  int64_t b, v, d;
+  int64_t stride_e, stride_cv, stride_cd;
+  int nrb, nvt, nsplit, nitems, items_per_xcd;
+  int stat_cols;
+  Softcap sc;
+};
+
+constexpr int kFwdWV = 4, kFwdWT = 4, kFwdNWV = 2, kFwdNWT = 2;
+
+template <typename T, bool ALIGNED, bool WANT_LA>
+__global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
+  using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, ALIGNED>;
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  // XCD-aware item id: workgroup ids that land on one XCD get consecutive items.
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  if (slot >= p.items_per_xcd) return;
+  const int item = xcd * p.items_per_xcd + slot;
+  if (item >= p.nitems) return;
+  const int rb = item / p.nsplit;
+  const int split = item % p.nsplit;
+  const int vt_begin = static_cast<int>((static_cast<int64_t>(p.nvt) * split) / p.nsplit);
+  const int vt_end = static_cast<int>((static_cast<int64_t>(p.nvt) * (split + 1)) / p.nsplit);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wv = wave / kFwdNWT;
+  const int wt = wave % kFwdNWT;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int64_t t0 = static_cast<int64_t>(rb) * Tile::TILE_T;
+
+  typename Tile::CLoader cl;
+  typename Tile::ELoader el;
+#pragma unroll
+  for (int q = 0; q < Tile::ELoader::NQ; ++q) {
+    const int64_t i = t0 + (tid >> 3) + q * Tile::ELoader::ROWSTEP;
+    const uint16_t* ptr = nullptr;
+    if (i < p.b) {
+      const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
+      ptr = p.e + row * p.stride_e;
+    }
+    el.ptr[q] = ptr;
+  }
+
+  float m2[kFwdWT], sum[kFwdWT];
+#pragma unroll
+  for (int ti = 0; ti < kFwdWT; ++ti) {
+    m2[ti] = -INFINITY;
+    sum[ti] = 0.0f;
+  }
+
+  // rows of this lane that exist (needed for the optional column average only)
+  float tok_ok[kFwdWT];
+#pragma unroll
+  for (int ti = 0; ti < kFwdWT; ++ti)
+    tok_ok[ti] = (t0 + wt * 128 + ti * 32 + l32 < p.b) ? 1.0f : 0.0f;
+
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int64_t v0 = static_cast<int64_t>(vt) * Tile::TILE_V;
+#pragma unroll
+    for (int q = 0; q < Tile::CLoader::NQ; ++q) {
+      const int64_t vr = v0 + (tid >> 3) + q * Tile::CLoader::ROWSTEP;
+      cl.ptr[q] = (vr < p.v) ? p.c + vr * p.stride_cv : nullptr;
+    }
+
+    f32x16 acc[kFwdWV][kFwdWT];
+    Tile::run(acc, cl, el, smem, static_cast<int>(p.d), p.stride_cd);
+
+    // ---- epilogue: bias, soft-cap, mask, online max / sum-exp ---------------------------------
+    const int64_t vw0 = v0 + wv * 128;  // first class of this wave
+    const bool ragged = (vw0 + 128 > p.v);
+#pragma unroll
+    for (int vi = 0; vi < kFwdWV; ++vi) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t vg = vw0 + vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        float bias = 0.0f;
+        if (p.bias != nullptr && vg < p.v) bias = Elem<T>::to_float(p.bias[vg]);
+        const bool dead = ragged && (vg >= p.v);
+#pragma unroll
+        for (int ti = 0; ti < kFwdWT; ++ti) {
+          float th;
+          float s2 = softcap_log2(p.sc, acc[vi][ti][r] + bias, th);
+          acc[vi][ti][r] = dead ? -INFINITY : s2;
+        }
+      }
+    }
+
+    if (WANT_LA) {
+      // column sums over the rows of this wave, in natural-log units
+      const float inv_b = kLn2 / static_cast<float>(p.b);
+#pragma unroll
+      for (int vi = 0; vi < kFwdWV; ++vi) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t vg = vw0 + vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          float colsum = 0.0f;
+#pragma unroll
+          for (int ti = 0; ti < kFwdWT; ++ti) {
+            float x = acc[vi][ti][r];
+            colsum += (vg < p.v) ? x * tok_ok[ti] : 0.0f;
+          }
+#pragma unroll
+          for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
+          if (l32 == 0 && vg < p.v) unsafeAtomicAdd(p.logit_avg + vg, colsum * inv_b);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int ti = 0; ti < kFwdWT; ++ti) {
+      float tm = -INFINITY;
+#pragma unroll
+      for (int vi = 0; vi < kFwdWV; ++vi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tm = fmaxf(tm, acc[vi][ti][r]);
+
+      if (p.tile_max != nullptr) {
+        // max over the 32 rows x 128 classes of this (wave, ti) cell
+        const float cell = wave_max(tm);
+        const int64_t srow = (t0 + wt * 128 + ti * 32) / CCE_STAT_ROWS;
+        const int64_t scol = vw0 / CCE_STAT_COLS;
+        if (lane == 0 && (t0 + wt * 128 + ti * 32) < p.b && vw0 < p.v)
+          p.tile_max[srow * p.stat_cols + scol] = cell * kLn2;
+      }
+
+      const float mn = fmaxf(m2[ti], tm);
+      const float ms = (mn == -INFINITY) ? 0.0f : mn;
+      float part = 0.0f;
+#pragma unroll
+      for (int vi = 0; vi < kFwdWV; ++vi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part += __builtin_amdgcn_exp2f(acc[vi][ti][r] - ms);
+      sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + part;
+      m2[ti] = mn;
+    }
+  }
+
+  // ---- merge the two lane halves, then the two wave rows, and emit one partial per row -------
+  float2* stage = reinterpret_cast<float2*>(smem);  // [NWT][WT][32]
+#pragma unroll
+  for (int ti = 0; ti < kFwdWT; ++ti) {
+    const float om = __shfl_xor(m2[ti], 32, 64);
+    const float os = __shfl_xor(sum[ti], 32, 64);
+    const float mn = fmaxf(m2[ti], om);
+    const float ms = (mn == -INFINITY) ? 0.0f : mn;
+    sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + os * __builtin_amdgcn_exp2f(om - ms);
+    m2[ti] = mn;
+  }
+  if (wv == 1 && half == 0) {
+#pragma unroll
+    for (int ti = 0; ti < kFwdWT; ++ti) stage[(wt * kFwdWT + ti) * 32 + l32] = make_float2(m2[ti], sum[ti]);
+  }
+  __syncthreads();
+  if (wv == 0 && half == 0) {
+#pragma unroll
+    for (int ti = 0; ti < kFwdWT; ++ti) {
+      const float2 o = stage[(wt * kFwdWT + ti) * 32 + l32];
+      const float mn = fmaxf(m2[ti], o.x);
+      const float ms = (mn == -INFINITY) ? 0.0f : mn;
+      const float s = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + o.y * __builtin_amdgcn_exp2f(o.x - ms);
+      const int64_t i = t0 + wt * 128 + ti * 32 + l32;
+      if (i < p.b) p.partial[static_cast<int64_t>(split) * p.b + i] = make_float2(mn, s);
+    }
+  }
+}
+
+// lse[i] = ln(2) * (M + log2(sum_s sum_s * 2^(m_s - M))),  M = max_s m_s
+__global__ void lse_merge_kernel(const float2* partial, float* lse, int64_t b, int nsplit) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= b) return;
+  float m = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, partial[static_cast<int64_t>(s) * b + i].x);
+  float acc = 0.0f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float2 ps = partial[static_cast<int64_t>(s) * b + i];
+    acc += ps.y * exp2f(ps.x - m);
+  }
+  lse[i] = (m + log2f(acc)) * kLn2;
+}
+
+__global__ void fill_zero_kernel(float* p, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.0f;
+}
+
+// Spans per row block: enough items to fill the CUs, as few as possible beyond that
+// (each extra span re-reads the E block's share of L2 and writes one more partial).
+static int choose_nsplit(int nrb, int nvt) {
+  const int num_cu = 256;
+  int best = 1;
+  double best_cost = 1e300;
+  const int max_split = nvt < 64 ? nvt : 64;
+  for (int s = 1; s <= max_split; ++s) {
+    const int64_t items = static_cast<int64_t>(nrb) * s;
+    const int64_t rounds = (items + num_cu - 1) / num_cu;
+    const int tiles_per_item = (nvt + s - 1) / s;
+    const double cost = static_cast<double>(rounds) * tiles_per_item + 0.02 * s;
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
+template <typename T>
+static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipStream_t stream) {
+  using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, true>;
+  const int lds = Tile::LDS_BYTES;
+  const int grid = p.items_per_xcd * 8;
+  hipError_t err;
+#define CCE_LAUNCH_FWD(AL, LA)                                                                    \
+  do {                                                                                            \
+    auto kern = lse_forward_kernel<T, AL, LA>;                                                    \
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+    if (err != hipSuccess) return status_from_hip(err);                                           \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, p);                              \
+  } while (0)
+  if (aligned) {
+    if (want_la) CCE_LAUNCH_FWD(true, true); else CCE_LAUNCH_FWD(true, false);
+  } else {
+    if (want_la) CCE_LAUNCH_FWD(false, true); else CCE_LAUNCH_FWD(false, false);
+  }
+#undef CCE_LAUNCH_FWD
+  return status_from_hip(hipGetLastError());
+}
+
+}  // namespace cce
+
+using namespace cce;
+
+extern "C" int64_t cce_tile_stat_elems(int64_t b, int64_t v) {
+  if (b <= 0 || v <= 0) return 0;
+  return ((b + CCE_STAT_ROWS - 1) / CCE_STAT_ROWS) * ((v + CCE_STAT_COLS - 1) / CCE_STAT_COLS);
+}
+
+extern "C" int64_t cce_lse_forward_workspace_bytes(int64_t b, int64_t v, int64_t d) {
+  (void)d;
+  if (b <= 0 || v <= 0) return 0;
+  const int nrb = static_cast<int>((b + 255) / 256);
+  const int nvt = static_cast<int>((v + 255) / 256);
+  const int nsplit = choose_nsplit(nrb, nvt);
+  return static_cast<int64_t>(nsplit) * b * static_cast<int64_t>(sizeof(float2));
+}
+
+extern "C" int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_t* valids,
+                               float* lse, float* logit_avg, float* tile_max,
+                               void* workspace, int64_t workspace_bytes,
+                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                               float softcap, int dtype, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (b < 0 || v <= 0 || d <= 0 || n_rows < 0) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0) return CCE_OK;
+  if (e == nullptr || c == nullptr || lse == nullptr) return CCE_ERR_INVALID_ARGUMENT;
+  if (valids == nullptr && b > n_rows) return CCE_ERR_INVALID_ARGUMENT;
+  if (d > (1 << 30) || b > (int64_t(1) << 40) || v > (int64_t(1) << 31) - 512) return CCE_ERR_INVALID_ARGUMENT;
+  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+  const int64_t need = cce_lse_forward_workspace_bytes(b, v, d);
+  if (workspace == nullptr || workspace_bytes < need) return CCE_ERR_WORKSPACE_TOO_SMALL;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return CCE_ERR_MISALIGNED;
+
+  LseFwdParams p;
+  p.e = static_cast<const uint16_t*>(e);
+  p.c = static_cast<const uint16_t*>(c);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.valids = valids;
+  p.logit_avg = logit_avg;
+  p.tile_max = tile_max;
+  p.partial = static_cast<float2*>(workspace);
+  p.b = b;
+  p.v = v;
+  p.d = d;
+  p.stride_e = stride_e;
+  p.stride_cv = stride_cv;
+  p.stride_cd = stride_cd;
+  p.nrb = static_cast<int>((b + 255) / 256);
+  p.nvt = static_cast<int>((v + 255) / 256);
+  p.nsplit = choose_nsplit(p.nrb, p.nvt);
+  p.nitems = p.nrb * p.nsplit;
+  p.items_per_xcd = (p.nitems + 7) / 8;
+  p.stat_cols = static_cast<int>((v + CCE_STAT_COLS - 1) / CCE_STAT_COLS);
+  p.sc = make_softcap(softcap);
+
+  const bool aligned = aligned16(e) && aligned16(c) && (d % 8 == 0) && (stride_e % 8 == 0) &&
+                       (stride_cv % 8 == 0) && (stride_cd == 1);
+
+  if (logit_avg != nullptr) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(static_cast<unsigned>((v + 255) / 256)), dim3(256), 0, stream,
+                       logit_avg, v);
+  }
+  int st = (dtype == CCE_DTYPE_BF16) ? launch_lse_forward<BF16>(p, aligned, logit_avg != nullptr, stream)
+                                     : launch_lse_forward<F16>(p, aligned, logit_avg != nullptr, stream);
+  if (st != CCE_OK) return st;
+  hipLaunchKernelGGL(lse_merge_kernel, dim3(static_cast<unsigned>((b + 255) / 256)), dim3(256), 0, stream,
+                     p.partial, lse, b, p.nsplit);
+  return status_from_hip(hipGetLastError());
+}

@@ -1,0 +1,141 @@
+"""Launcher of the fused backward kernel
+(reference: cut_cross_entropy/cce_backward.py:346-521)."""
+
+from typing import Optional, Tuple
+
+import torch
+
+from cut_cross_entropy import _hip
+from cut_cross_entropy.cce_utils import filter_eps_or_none
+from cut_cross_entropy.utils import TensorInfo
+
+
+def cce_backward_kernel(
+    do: torch.Tensor,
+    dlse: Optional[torch.Tensor],
+    e: torch.Tensor,
+    e_info: TensorInfo,
+    c: torch.Tensor,
+    c_info: TensorInfo,
+    bias: Optional[torch.Tensor],
+    bias_info: Optional[TensorInfo],
+    lse: torch.Tensor,
+    valids: Optional[torch.Tensor],
+    softcap: Optional[float],
+    filter_eps: Optional[float],
+    targets: Optional[torch.Tensor] = None,
+    shift: int = 0,
+    vocab_ordering: Optional[torch.Tensor] = None,
+    grad_scale: float = 1.0,
+    accum_e_fp32: bool = False,
+    accum_c_fp32: bool = False,
+    filter_e_grad: bool = True,
+    filter_c_grad: bool = True,
+    reduce_e_grad: bool = False,
+    pg=None,
+    tile_max: Optional[torch.Tensor] = None,
+    target_offset: int = 0,
+    counters: Optional[torch.Tensor] = None,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Returns ``(de, dc, dbias)`` in the dtypes recorded in the ``*_info`` arguments; an
+    entry is ``None`` when that input does not require a gradient (reference :391-403,
+    :511-519).
+
+    ``do`` is one element (mean / sum reductions) or the per-position upstream gradient of
+    the whole batch, read at ``row + shift``; ``dlse`` likewise.  ``lse`` must be the global
+    log-sum-exp when ``c`` is a vocabulary shard.
+
+    Additions to the reference signature: ``tile_max`` (statistic of the forward pass that
+    lets whole tiles be dropped before their logits are recomputed), ``target_offset``
+    (first class of a vocabulary shard; the reference rebases ``targets`` on the host,
+    cce.py:193-205) and ``counters`` (uint64[4] device tensor accumulating tiles in the
+    grid / recomputed / with a dE product / with a dC product).  ``reduce_e_grad`` and
+    ``pg`` belong to the reference's all-reduce of dE and must be left unset here.
+    """
+    assert do.numel() in (e.size(0), 1)
+    assert c.size(1) == e.size(1)
+    assert lse.size(0) == e.size(0) or (valids is not None and lse.size(0) == valids.size(0))
+    assert e.ndim == 2 and c.ndim == 2 and e.is_contiguous()
+    if reduce_e_grad:
+        raise NotImplementedError("summing dE over vocabulary-parallel ranks is not part of this build")
+    _hip.require_gpu_tensor("e", e)
+    code = _hip.dtype_code(e.dtype)
+    lib = _hip.load()
+    dev = e.device
+
+    if targets is None:
+        # no one-hot term at all: every row gets a target that matches no class
+        targets = torch.full((e.size(0),), -1, dtype=torch.int64, device=dev)
+    targets = targets.to(torch.int64).contiguous()
+    assert targets.numel() == e.size(0)
+
+    do = do.to(torch.float32).contiguous().view(-1)
+    lse = lse.to(torch.float32).contiguous()
+    if dlse is not None:
+        dlse = dlse.to(torch.float32).contiguous().view(-1)
+        assert dlse.numel() == e.size(0)
+        if do.numel() > 1:
+            assert dlse.size() == do.size()
+
+    de_dtype = torch.float32 if accum_e_fp32 else e.dtype
+    dc_dtype = torch.float32 if accum_c_fp32 else c.dtype
+    de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
+    dc = torch.zeros_like(c, dtype=dc_dtype) if c_info.requires_grad else None
+    dbias = None
+    if bias is not None:
+        assert bias_info is not None
+        bias = bias.to(e.dtype).contiguous()
+        if bias_info.requires_grad:
+            dbias = torch.zeros((bias.numel(),), dtype=torch.float32, device=dev)
+    if de is not None:
+        assert de.stride() == e.stride()
+    if dc is not None:
+        assert dc.stride() == c.stride()
+
+    if valids is not None:
+        assert valids.ndim == 1 and valids.dtype == torch.int32
+        valids = valids.contiguous()
+        B = valids.size(0)
+    else:
+        B = e.size(0)
+
+    if vocab_ordering is not None:
+        assert vocab_ordering.ndim == 1
+        assert vocab_ordering.numel() == c.size(0)
+        assert vocab_ordering.stride(0) == 1
+        vocab_ordering = vocab_ordering.to(torch.int32)
+    if tile_max is not None:
+        assert tile_max.dtype == torch.float32 and tile_max.is_contiguous()
+        assert tile_max.numel() == lib.cce_tile_stat_elems(B, c.size(0))
+    if counters is not None:
+        assert counters.dtype in (torch.int64, torch.uint64) and counters.numel() >= _hip.NUM_COUNTERS
+        assert counters.is_contiguous() and counters.device == dev
+
+    if B > 0 and (de is not None or dc is not None or dbias is not None):
+        with torch.cuda.device(dev):
+            status = lib.cce_backward(
+                e.data_ptr(), c.data_ptr(), _hip.ptr(bias),
+                lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
+                _hip.ptr(valids), _hip.ptr(vocab_ordering), targets.data_ptr(),
+                _hip.ptr(tile_max),
+                _hip.ptr(de), _hip.ptr(dc), _hip.ptr(dbias),
+                None, 0, _hip.ptr(counters),
+                e.size(0), B, c.size(0), e.size(1),
+                e.stride(0), c.stride(0), c.stride(1),
+                float(grad_scale), filter_eps_or_none(filter_eps),
+                1 if filter_e_grad else 0, 1 if filter_c_grad else 0,
+                1 if de_dtype == torch.float32 else 0, 1 if dc_dtype == torch.float32 else 0,
+                int(shift), int(target_offset),
+                float(softcap) if softcap is not None else 0.0, code,
+                _hip.current_stream_ptr(dev),
+            )
+        _hip.check(status, "cce_backward")
+
+    if dbias is not None:
+        assert bias_info is not None
+        dbias = dbias.to(dtype=bias_info.dtype)
+    if dc is not None:
+        dc = dc.to(dtype=c_info.dtype)
+    if de is not None:
+        de = de.to(dtype=e_info.dtype)
+    return de, dc, dbias

@@ -1,0 +1,161 @@
+"""Parity of the three HIP kernels, called through the C ABI, against the CPU oracle."""
+
+import ctypes
+
+import pytest
+import torch
+
+from _util import IGNORE_INDEX, assert_no_worse, autograd_grads, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(256, 512, 128), (255, 507, 128), (255, 507, 123), (300, 1000, 72), (64, 130, 64)]
+
+
+def _lib():
+    from cut_cross_entropy import _hip
+
+    return _hip.load()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_lse_forward_abi(dtype, softcap, has_bias, shape):
+    """cce_lse_forward vs logsumexp of the dense logits (reference tests/test_cce_lse.py:23-63)."""
+    from oracle import dense_lce
+
+    N, V, D = shape
+    e, c, _, bias = make_inputs(N, V, D, dtype, seed=1, bias=has_bias)
+    gt = dense_lce.dense_lse(e, c, bias, softcap, compute_dtype=torch.float64)
+    ref = dense_lce.dense_lse(e, c, bias, softcap, compute_dtype=dtype)
+
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    ed, cd = e.to(dev), c.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    lse = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    la = torch.empty((V,), dtype=torch.float32, device=dev)
+    tm = torch.empty((lib.cce_tile_stat_elems(N, V),), dtype=torch.float32, device=dev)
+    ws_bytes = lib.cce_lse_forward_workspace_bytes(N, V, D)
+    ws = torch.empty((ws_bytes // 8 + 1,), dtype=torch.int64, device=dev)
+    st = lib.cce_lse_forward(
+        ed.data_ptr(), cd.data_ptr(), bd.data_ptr() if bd is not None else None, None,
+        lse.data_ptr(), la.data_ptr(), tm.data_ptr(), ws.data_ptr(), ws.numel() * 8,
+        N, N, V, D, ed.stride(0), cd.stride(0), cd.stride(1),
+        softcap or 0.0, 0 if dtype == torch.bfloat16 else 1,
+        torch.cuda.current_stream().cuda_stream,
+    )
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    assert_no_worse(gt, ref, lse, 1e-5 if dtype == torch.float16 else 2e-5, "lse")
+
+    # column average of the (soft-capped) logits
+    logits = dense_lce._dense_logits(e, c, bias, softcap, torch.float64)
+    assert torch.allclose(la.cpu().double(), logits.mean(0), atol=2e-2, rtol=2e-2)
+
+    # tile statistic: max soft-capped logit per 32-row x 128-class cell
+    nr, nc = (N + 31) // 32, (V + 127) // 128
+    want = torch.full((nr, nc), float("-inf"), dtype=torch.float64)
+    for r in range(nr):
+        for cc in range(nc):
+            want[r, cc] = logits[r * 32 : (r + 1) * 32, cc * 128 : (cc + 1) * 128].max()
+    got = tm.cpu().double().view(nr, nc)
+    assert (got >= want - 0.05).all() and (got <= want + 0.05).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (255, 507, 123), (100, 300, 520)])
+def test_indexed_neg_dot_abi(dtype, softcap, has_bias, shape):
+    """cce_indexed_neg_dot vs the explicit gather-dot (reference tests/test_cce_indexed_dot.py:11-66).
+    D = 520 > 256 with a bias checks that the bias is subtracted exactly once."""
+    from oracle import dense_lce
+
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=2, bias=has_bias)
+    gt = dense_lce.dense_indexed_neg_dot(e, c, t, bias, softcap, torch.float64)
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    ed, cd, td = e.to(dev), c.to(dev), t.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    out = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    st = lib.cce_indexed_neg_dot(
+        ed.data_ptr(), cd.data_ptr(), td.data_ptr(), bd.data_ptr() if bd is not None else None, None,
+        out.data_ptr(), N, N, V, D, ed.stride(0), cd.stride(0), cd.stride(1), 0, 0,
+        softcap or 0.0, 0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream,
+    )
+    assert st == 0
+    torch.cuda.synchronize()
+    # products are exact in fp32, only the summation order differs
+    assert torch.allclose(out.cpu().double(), gt, atol=1e-5, rtol=1e-5)
+
+
+def _run_backward_abi(e, c, t, bias, valids, lse, d_out, d_lse, softcap, shift, grad_scale, filter_eps,
+                      fp32_accum, dtype, order=None):
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, D = e.shape
+    V = c.shape[0]
+    ed, cd, td = e.to(dev), c.to(dev), t.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    vd = valids.to(dev) if valids is not None else None
+    B = valids.numel() if valids is not None else N
+    lsed = lse.float().to(dev)
+    dod = d_out.float().to(dev).contiguous()
+    dld = d_lse.float().to(dev).contiguous() if d_lse is not None else None
+    od = order.to(dev) if order is not None else None
+    gdt = torch.float32 if fp32_accum else dtype
+    de = torch.zeros((N, D), dtype=gdt, device=dev)
+    dc = torch.zeros((V, D), dtype=gdt, device=dev)
+    db = torch.zeros((V,), dtype=torch.float32, device=dev) if bias is not None else None
+    counters = torch.zeros((4,), dtype=torch.int64, device=dev)
+    p = lambda x: x.data_ptr() if x is not None else None
+    st = lib.cce_backward(
+        p(ed), p(cd), p(bd), p(lsed), p(dod), 1 if dod.numel() == 1 else 0, p(dld),
+        p(vd), p(od), p(td), None, p(de), p(dc), p(db), None, 0, p(counters),
+        N, B, V, D, ed.stride(0), cd.stride(0), cd.stride(1),
+        grad_scale, -1.0 if filter_eps is None else filter_eps, 1, 1,
+        1 if fp32_accum else 0, 1 if fp32_accum else 0, shift, 0,
+        softcap or 0.0, 0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream,
+    )
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    return de.cpu(), dc.cpu(), (db.cpu() if db is not None else None), counters.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("with_dlse", [False, True])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (255, 507, 123), (200, 700, 72)])
+def test_backward_abi_exact(dtype, softcap, has_bias, with_dlse, shape):
+    """cce_backward without filtering, fp32 accumulation, vs the closed-form dense gradients."""
+    from oracle import dense_lce
+
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=3, bias=has_bias, invalid_frac=0.2)
+    valids = dense_lce.build_flat_valids(t, IGNORE_INDEX, 0)
+    g = torch.Generator().manual_seed(7)
+    d_out = torch.randn((N,), generator=g)
+    d_lse = torch.randn((N,), generator=g) * 0.1 if with_dlse else None
+    rows = valids.long()
+    lse = dense_lce.dense_lse(e[rows], c, bias, softcap, torch.float64)
+
+    gt = dense_lce.dense_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, torch.float64)
+    ref = autograd_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, dtype)
+    de, dc, db, counters = _run_backward_abi(e, c, t, bias, valids, lse, d_out, d_lse, softcap, 0, 0.5,
+                                             None, True, dtype)
+    tol = 2e-3
+    assert_no_worse(gt[0], ref[0], de, tol, "dE")
+    assert_no_worse(gt[1], ref[1], dc, tol, "dC")
+    if has_bias:
+        assert_no_worse(gt[2], ref[2], db, tol, "dBias")
+    # ignored rows get exactly zero gradient
+    ignored = torch.ones(N, dtype=torch.bool)
+    ignored[rows] = False
+    assert (de[ignored] == 0).all()
+    nt = ((valids.numel() + 127) // 128) * ((V + 127) // 128)
+    assert counters.tolist() == [nt, nt, nt, nt]
