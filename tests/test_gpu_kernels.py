@@ -148,11 +148,12 @@ def test_backward_abi_exact(dtype, softcap, has_bias, with_dlse, shape):
     ref = autograd_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, dtype)
     de, dc, db, counters = _run_backward_abi(e, c, t, bias, valids, lse, d_out, d_lse, softcap, 0, 0.5,
                                              None, True, dtype)
-    tol = 2e-3
-    assert_no_worse(gt[0], ref[0], de, tol, "dE")
-    assert_no_worse(gt[1], ref[1], dc, tol, "dC")
+    # 1e-2 relative per element (bf16 rounding of dz) plus a small absolute floor
+    tol, rel = 2e-3, 1e-2
+    assert_no_worse(gt[0], ref[0], de, tol, "dE", rel)
+    assert_no_worse(gt[1], ref[1], dc, tol, "dC", rel)
     if has_bias:
-        assert_no_worse(gt[2], ref[2], db, tol, "dBias")
+        assert_no_worse(gt[2], ref[2], db, tol, "dBias", rel)
     # ignored rows get exactly zero gradient
     ignored = torch.ones(N, dtype=torch.bool)
     ignored[rows] = False

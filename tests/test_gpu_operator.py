@@ -1,0 +1,172 @@
+"""Operator-level parity: cut_cross_entropy.linear_cross_entropy (HIP kernels) against the CPU
+oracle, with the reference's own accuracy criterion and parameter grid
+(reference tests/test_cce_loss_forward.py:44-108, tests/test_cce_loss_backward.py:79-227)."""
+
+import pytest
+import torch
+
+from _util import IGNORE_INDEX, assert_no_worse, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(256, 512, 128), (252, 507, 128), (252, 507, 123)]
+TOL = {torch.float16: 1e-3, torch.bfloat16: 1e-2}
+
+
+def _oracle_loss(e, c, targets, bias, softcap, shift, reduction, z_loss, compute_dtype, want_grads):
+    """Loss (and gradients) of the dense oracle with leaves in ``compute_dtype``; the test
+    objective mirrors the reference test: mean of the per-token loss (+ z-loss of the lse)."""
+    from oracle import dense_lce
+
+    el = e.detach().to(compute_dtype).requires_grad_(want_grads)
+    cl = c.detach().to(compute_dtype).requires_grad_(want_grads)
+    bl = bias.detach().to(compute_dtype).requires_grad_(want_grads) if bias is not None else None
+    loss, lse = dense_lce.dense_linear_cross_entropy(
+        el, cl, targets, bl, IGNORE_INDEX, softcap, reduction, shift, return_lse=z_loss
+    )
+    out = loss
+    if want_grads:
+        obj = loss
+        if reduction == "sum":
+            obj = obj / (targets[..., shift:] != IGNORE_INDEX).count_nonzero()
+        obj = obj.mean()
+        if z_loss:
+            obj = obj + dense_lce.compute_z_loss(lse, targets, shift)
+        obj.backward()
+        return out.detach(), (el.grad, cl.grad, bl.grad if bl is not None else None)
+    return out.detach(), None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [True, False])
+@pytest.mark.parametrize("shift", [0, 2])
+@pytest.mark.parametrize("invalids", [False, True])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_loss_forward(dtype, softcap, has_bias, shift, invalids, shape):
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=11, bias=has_bias, invalid_frac=0.2 if invalids else 0.0)
+    e = e.view(4, -1, D)
+    t = t.view(4, -1)
+    gt, _ = _oracle_loss(e, c, t, bias, softcap, shift, "none", False, torch.float64, False)
+    ref, _ = _oracle_loss(e, c, t, bias, softcap, shift, "none", False, dtype, False)
+
+    dev = torch.device("cuda:0")
+    got = linear_cross_entropy(
+        e.to(dev), c.to(dev), t.to(dev), bias=bias.to(dev) if has_bias else None,
+        softcap=softcap, shift=shift, reduction="none", impl="cce",
+    )
+    assert got.dtype == torch.float32
+    assert got.shape == (4, N // 4 - shift)
+    assert_no_worse(gt, ref, got, TOL[dtype], "loss")
+    # bit-exact masking: ignored positions are exactly zero
+    ign = t[..., shift:] == IGNORE_INDEX
+    assert (got.cpu()[ign] == 0).all()
+
+
+@pytest.mark.parametrize("impl", ["cce", "cce_exact", "cce_kahan_full_c", "cce_kahan_full_e", "cce_kahan"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("shift", [False, True])
+@pytest.mark.parametrize("invalids", [False, True])
+@pytest.mark.parametrize("reduction", ["none", "mean", "sum"])
+@pytest.mark.parametrize("z_loss", [True, False])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (252, 507, 123)])
+def test_loss_backward(impl, dtype, softcap, has_bias, shift, invalids, reduction, z_loss, shape):
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import compute_z_loss
+
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=12, bias=has_bias, invalid_frac=0.2 if invalids else 0.0)
+    e = e.view(4, -1, D)
+    t = t.view(4, -1)
+    sh = int(shift)
+    _, gt = _oracle_loss(e, c, t, bias, softcap, sh, reduction, z_loss, torch.float64, True)
+    _, ref = _oracle_loss(e, c, t, bias, softcap, sh, reduction, z_loss, dtype, True)
+
+    dev = torch.device("cuda:0")
+    ed = e.to(dev).requires_grad_(True)
+    cd = c.to(dev).requires_grad_(True)
+    bd = bias.to(dev).requires_grad_(True) if has_bias else None
+    td = t.to(dev)
+    out = linear_cross_entropy(ed, cd, td, bias=bd, softcap=softcap, shift=shift, reduction=reduction,
+                               impl=impl, return_lse=z_loss)
+    loss, lse = out if z_loss else (out, None)
+    if reduction == "sum":
+        loss = loss / (td[..., sh:] != IGNORE_INDEX).count_nonzero()
+    loss = loss.mean()
+    if z_loss:
+        loss = loss + compute_z_loss(lse, td, shift)
+    loss.backward()
+
+    assert ed.grad.dtype == dtype and cd.grad.dtype == dtype
+    names = ["dE", "dC", "dBias"]
+    got = [ed.grad, cd.grad, bd.grad if has_bias else None]
+    for name, g_gt, g_ref, g in zip(names, gt, ref, got):
+        if g is None:
+            continue
+        assert_no_worse(g_gt, g_ref, g, TOL[dtype], f"{impl} {name}")
+
+
+@pytest.mark.parametrize(
+    "compute_de,compute_dc,compute_dbias",
+    [(True, False, True), (False, True, False), (False, False, True), (True, True, False)],
+)
+def test_loss_partials(compute_de, compute_dc, compute_dbias):
+    """Only the inputs that require a gradient receive one (reference test_loss_partials)."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, V, D = 256, 512, 128
+    e, c, t, bias = make_inputs(N, V, D, torch.bfloat16, seed=13, bias=True)
+    dev = torch.device("cuda:0")
+    ed = e.view(4, -1, D).to(dev).requires_grad_(compute_de)
+    cd = c.to(dev).requires_grad_(compute_dc)
+    bd = bias.to(dev).requires_grad_(compute_dbias)
+    loss = linear_cross_entropy(ed, cd, t.view(4, -1).to(dev), bias=bd, reduction="mean")
+    loss.backward()
+    assert (ed.grad is not None) == compute_de
+    assert (cd.grad is not None) == compute_dc
+    assert (bd.grad is not None) == compute_dbias
+
+
+def test_all_ignored_batch():
+    """mean over zero valid tokens: NaN loss like F.cross_entropy, zero gradients, no exception."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    dev = torch.device("cuda:0")
+    e = torch.randn((2, 8, 64), device=dev, dtype=torch.bfloat16, requires_grad=True)
+    c = torch.randn((96, 64), device=dev, dtype=torch.bfloat16, requires_grad=True)
+    t = torch.full((2, 8), IGNORE_INDEX, device=dev)
+    loss = linear_cross_entropy(e, c, t)
+    assert torch.isnan(loss)
+    loss.backward()
+    assert (e.grad == 0).all() and (c.grad == 0).all()
+    none = linear_cross_entropy(e, c, t, reduction="none")
+    assert (none == 0).all() and none.shape == (2, 8)
+
+
+def test_module_and_enum():
+    from cut_cross_entropy import LinearCrossEntropy, LinearCrossEntropyImpl, linear_cross_entropy
+
+    e, c, t, _ = make_inputs(128, 256, 64, torch.bfloat16, seed=14)
+    dev = torch.device("cuda:0")
+    e, c, t = e.to(dev), c.to(dev), t.to(dev)
+    a = LinearCrossEntropy(softcap=10.0, impl=LinearCrossEntropyImpl.CCE_EXACT)(e, c, t)
+    b = linear_cross_entropy(e, c, t, softcap=10.0, impl="cce_exact")
+    assert torch.equal(a, b)
+    d = linear_cross_entropy(e, c, t, softcap=10.0, impl="torch_compile")
+    assert torch.allclose(a, d, rtol=1e-2, atol=1e-2)
+
+
+def test_deterministic_forward():
+    from cut_cross_entropy import linear_cross_entropy
+
+    e, c, t, _ = make_inputs(512, 1024, 128, torch.bfloat16, seed=15)
+    dev = torch.device("cuda:0")
+    e, c, t = e.to(dev), c.to(dev), t.to(dev)
+    a = linear_cross_entropy(e, c, t, reduction="none")
+    b = linear_cross_entropy(e, c, t, reduction="none")
+    assert torch.equal(a, b)
