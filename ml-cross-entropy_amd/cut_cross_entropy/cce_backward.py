@@ -48,8 +48,8 @@ def cce_backward_kernel(
     Additions to the reference signature: ``tile_max`` (statistic of the forward pass that
     lets whole tiles be dropped before their logits are recomputed), ``target_offset``
     (first class of a vocabulary shard; the reference rebases ``targets`` on the host,
-    cce.py:193-205) and ``counters`` (uint64[4] device tensor accumulating tiles in the
-    grid / recomputed / with a dE product / with a dC product).  ``reduce_e_grad`` and
+    cce.py:193-205) and ``counters`` (uint64[4] device tensor accumulating 32 x 32 sub-tiles in the
+    plane / recomputed by the dE pass / with a dE product / with a dC product).  ``reduce_e_grad`` and
     ``pg`` belong to the reference's all-reduce of dE and must be left unset here.
     """
     assert do.numel() in (e.size(0), 1)
@@ -112,6 +112,8 @@ def cce_backward_kernel(
         assert counters.is_contiguous() and counters.device == dev
 
     if B > 0 and (de is not None or dc is not None or dbias is not None):
+        ws_bytes = lib.cce_backward_workspace_bytes(B, c.size(0), e.size(1))
+        workspace = torch.empty((max(ws_bytes, 8) // 8 + 1,), dtype=torch.int64, device=dev)
         with torch.cuda.device(dev):
             status = lib.cce_backward(
                 e.data_ptr(), c.data_ptr(), _hip.ptr(bias),
@@ -119,7 +121,7 @@ def cce_backward_kernel(
                 _hip.ptr(valids), _hip.ptr(vocab_ordering), targets.data_ptr(),
                 _hip.ptr(tile_max),
                 _hip.ptr(de), _hip.ptr(dc), _hip.ptr(dbias),
-                None, 0, _hip.ptr(counters),
+                workspace.data_ptr(), workspace.numel() * 8, _hip.ptr(counters),
                 e.size(0), B, c.size(0), e.size(1),
                 e.stride(0), c.stride(0), c.stride(1),
                 float(grad_scale), filter_eps_or_none(filter_eps),
