@@ -265,6 +265,187 @@ struct LogitTile {
   }
 };
 
+// ---------------------------------------------------------------------------------------------
+// Fast logit tile for the common case (16-byte aligned rows, unit column stride, D % 32 == 0).
+//
+// Differences to LogitTile: 32 reduction columns per LDS stage (64-byte rows, chunk swizzle with
+// (row >> 2) & 3), branch-free loads (a row outside the matrix is clamped to the last valid row:
+// its logits are discarded by the caller), and the global loads for stage k + 2 are issued before
+// the MFMAs of stage k, so two stages of HBM / L2 latency are hidden behind compute.
+// `lds` must hold 2 * (TILE_V + TILE_T) * 64 bytes.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFastBK = 32;
+constexpr int kFastRowBytes = 64;
+
+template <int ROWS, int NT>
+struct FastLoader {
+  static constexpr int NQ = ROWS * 4 / NT;
+  static constexpr int ROWSTEP = NT / 4;
+  static_assert(ROWS * 4 % NT == 0, "tile rows must divide evenly over the threads");
+  static_assert(ROWSTEP % 16 == 0, "swizzle must not depend on q");
+  const uint16_t* ptr[NQ];  // row base + this thread's 8-element chunk; always a readable address
+  struct Regs {
+    uint4 v[NQ];
+  };
+
+  __device__ __forceinline__ Regs load(int k0) const {
+    Regs r;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) r.v[q] = *reinterpret_cast<const uint4*>(ptr[q] + k0);
+    return r;
+  }
+  static __device__ __forceinline__ void store(const Regs& r, unsigned char* lds) {
+    const int row0 = threadIdx.x >> 2;
+    const int chunk = (threadIdx.x & 3) ^ ((row0 >> 2) & 3);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+      *reinterpret_cast<uint4*>(lds + (row0 + q * ROWSTEP) * kFastRowBytes + (chunk << 4)) = r.v[q];
+  }
+};
+
+template <typename T, int WV, int WT, int NWV, int NWT>
+struct FastLogitTile {
+  static constexpr int TILE_V = 32 * WV * NWV;
+  static constexpr int TILE_T = 32 * WT * NWT;
+  static constexpr int NT = 64 * NWV * NWT;
+  static constexpr int STAGE_BYTES = (TILE_V + TILE_T) * kFastRowBytes;
+  static constexpr int LDS_BYTES = 3 * STAGE_BYTES;
+  using CLoader = FastLoader<TILE_V, NT>;
+  using ELoader = FastLoader<TILE_T, NT>;
+  using vec8 = typename Elem<T>::vec8;
+
+  struct Frags {
+    vec8 a[WV];
+    vec8 b[WT];
+  };
+
+  // MFMA operands of one 16-column step: WV class fragments and WT row fragments of this wave.
+  static __device__ __forceinline__ Frags read_frags(const unsigned char* lds, int stage_off, int kk, int coff0,
+                                                     int eoff0, int sw, int half) {
+    Frags f;
+    const int chunk = (((kk * 2 + half) ^ sw) << 4);
+    const unsigned char* cb = lds + stage_off + coff0 + chunk;
+    const unsigned char* eb = lds + stage_off + eoff0 + chunk;
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+      f.a[vi] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(cb + vi * 32 * kFastRowBytes));
+#pragma unroll
+    for (int ti = 0; ti < WT; ++ti)
+      f.b[ti] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(eb + ti * 32 * kFastRowBytes));
+    return f;
+  }
+
+  static __device__ __forceinline__ void mma(f32x16 (&acc)[WV][WT], const Frags& f) {
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
+  }
+
+  // Issue order of one stage: the memory instructions are spread evenly between the MFMAs, so that
+  // the matrix pipe never waits for a burst of loads to issue.  First half: the global loads and the
+  // fragment reads of step 1; second half: the LDS stores and the fragment reads of the next stage.
+  template <int FIRST_MASK>
+  static __device__ __forceinline__ void interleave_half() {
+    constexpr int kMfma = 0x008, kDsRead = 0x100;
+    constexpr int nmem = CLoader::NQ + ELoader::NQ;  // global loads = LDS stores per stage
+    constexpr int nfrag = WV + WT;                    // fragment reads per step
+    constexpr int nmma = WV * WT;
+    constexpr int total = nmem + nfrag;
+#pragma unroll
+    for (int i = 0; i < nmma; ++i) {
+      __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+#pragma unroll
+      for (int j = i * total / nmma; j < (i + 1) * total / nmma; ++j) {
+        if (j < nmem) __builtin_amdgcn_sched_group_barrier(FIRST_MASK, 1, 0);
+        else __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+      }
+    }
+  }
+  static __device__ __forceinline__ void interleave() {
+    interleave_half<0x020>();  // VMEM reads
+    interleave_half<0x200>();  // DS writes
+  }
+
+  // Software pipeline, one barrier per 32-column stage s (LDS ring of three stages, two register
+  // sets for data in flight, two fragment sets):
+  //     issue global loads of stage s + 3          -> register set (s + 1) % 2
+  //     read fragments (s, step 1); MFMAs (s, step 0)
+  //     LDS[(s + 2) % 3] <- register set s % 2      (stage s + 2, issued one and a half trips ago)
+  //     read fragments (s + 1, step 0); MFMAs (s, step 1)
+  //     barrier
+  // Every LDS read is issued a full MFMA group before its use, every global load about two stages
+  // before its LDS store.  Prefetches past the last stage re-read it (never consumed), so the loop
+  // has no branches.
+  static __device__ __forceinline__ void run(f32x16 (&acc)[WV][WT], const CLoader& cl, const ELoader& el,
+                                             unsigned char* lds, int D) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wv = wave / NWT;
+    const int wt = wave % NWT;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int sw = (l32 >> 2) & 3;
+    const int coff0 = (wv * WV * 32 + l32) * kFastRowBytes;
+    const int eoff0 = (TILE_V + wt * WT * 32 + l32) * kFastRowBytes;
+
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[vi][ti][r] = 0.0f;
+
+    const int nk = D / kFastBK;
+    const int last = (nk - 1) * kFastBK;
+    typename CLoader::Regs rc0 = cl.load(0);
+    typename ELoader::Regs re0 = el.load(0);
+    typename CLoader::Regs rc1 = cl.load(min(kFastBK, last));
+    typename ELoader::Regs re1 = el.load(min(kFastBK, last));
+    CLoader::store(rc0, lds);
+    ELoader::store(re0, lds + TILE_V * kFastRowBytes);
+    rc0 = cl.load(min(2 * kFastBK, last));
+    re0 = el.load(min(2 * kFastBK, last));
+    CLoader::store(rc1, lds + STAGE_BYTES);
+    ELoader::store(re1, lds + STAGE_BYTES + TILE_V * kFastRowBytes);
+    __syncthreads();
+
+    int o0 = 0, o1 = STAGE_BYTES, o2 = 2 * STAGE_BYTES;  // LDS offsets of stages s, s + 1, s + 2
+    Frags f0 = read_frags(lds, o0, 0, coff0, eoff0, sw, half);
+    Frags f1;
+
+#define CCE_FAST_STAGE(S, RC_NEW, RE_NEW, RC_OLD, RE_OLD)                                        \
+  do {                                                                                            \
+    const int kn = min(((S) + 3) * kFastBK, last);                                                \
+    RC_NEW = cl.load(kn);                                                                         \
+    RE_NEW = el.load(kn);                                                                         \
+    f1 = read_frags(lds, o0, 1, coff0, eoff0, sw, half);                                          \
+    mma(acc, f0);                                                                                 \
+    CLoader::store(RC_OLD, lds + o2);                                                             \
+    ELoader::store(RE_OLD, lds + o2 + TILE_V * kFastRowBytes);                                    \
+    f0 = read_frags(lds, o1, 0, coff0, eoff0, sw, half);                                          \
+    mma(acc, f1);                                                                                 \
+    interleave();                                                                                 \
+    __syncthreads();                                                                              \
+    const int t = o0;                                                                             \
+    o0 = o1;                                                                                      \
+    o1 = o2;                                                                                      \
+    o2 = t;                                                                                       \
+  } while (0)
+
+    const int pairs = nk >> 1;
+#pragma unroll 1
+    for (int pi = 0; pi < pairs; ++pi) {
+      CCE_FAST_STAGE(2 * pi, rc1, re1, rc0, re0);
+      CCE_FAST_STAGE(2 * pi + 1, rc0, re0, rc1, re1);
+    }
+    if (nk & 1) {
+      CCE_FAST_STAGE(nk - 1, rc1, re1, rc0, re0);
+    }
+#undef CCE_FAST_STAGE
+  }
+};
+
 inline int status_from_hip(hipError_t e) { return e == hipSuccess ? CCE_OK : static_cast<int>(e); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

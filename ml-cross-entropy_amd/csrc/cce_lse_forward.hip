@@ -31,12 +31,56 @@ struct LseFwdParams {
   Softcap sc;
 };
 
-constexpr int kFwdWV = 4, kFwdWT = 4, kFwdNWV = 2, kFwdNWT = 2;
+// 8 waves (two per SIMD, so that one wave's LDS and global traffic issues in the shadow of the
+// other's MFMAs), 2 x 4: each wave owns 128 classes x 64 rows of the 256 x 256 tile.
+constexpr int kFwdWV = 4, kFwdWT = 2, kFwdNWV = 2, kFwdNWT = 4;
+constexpr int kFwdThreads = 64 * kFwdNWV * kFwdNWT;
+constexpr int kFwdTile = 256;
+static_assert(32 * kFwdWV * kFwdNWV == kFwdTile && 32 * kFwdWT * kFwdNWT == kFwdTile, "tile is 256 x 256");
+static_assert(32 * kFwdWV == CCE_STAT_COLS, "one statistic cell per (wave, 32-row block)");
 
-template <typename T, bool ALIGNED, bool WANT_LA>
-__global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
+constexpr int kFwdBiasBytes = 2 * 256 * 4;  // two tiles' worth of per-class addends (double-buffered)
+
+// Soft-capped logits (log2 domain) of one 32-row column block of a wave: 4 class blocks x 16 registers.
+// GENERAL adds a per-class addend staged in LDS: the bias (or 0), or -inf for a class past the end of
+// the vocabulary, which is masked AFTER soft-capping (soft-capping -inf would give -softcap, not -inf).
+// The plain variant is straight-line code with no loads.
+template <bool GENERAL>
+__device__ __forceinline__ float column_block_logits(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
+                                                     const float* addend, int half, float (&s2)[kFwdWV][16]) {
+  float tm = -INFINITY;
+#pragma unroll
+  for (int vi = 0; vi < kFwdWV; ++vi) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float x = acc[vi][ti][r];
+      float th;
+      if (GENERAL) {
+        const float add = addend[vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
+        const bool dead = (add == -INFINITY);
+        const float y = softcap_log2(sc, dead ? 0.0f : x + add, th);
+        s2[vi][r] = dead ? -INFINITY : y;
+      } else {
+        s2[vi][r] = softcap_log2(sc, x, th);
+      }
+      tm = fmaxf(tm, s2[vi][r]);
+    }
+  }
+  return tm;
+}
+
+// Kernel variants:
+//   FAST     rows 16-byte aligned, unit column stride, D % 32 == 0: software-pipelined main loop
+//   ALIGNED  (generic main loop only) 16-byte vector loads are legal
+//   GENERAL  a bias is present or V is not a multiple of the tile: per-class addend / mask from LDS
+//   WANT_LA  also accumulate the column average of the logits (needs GENERAL)
+template <typename T, bool FAST, bool ALIGNED, bool GENERAL, bool WANT_LA>
+__global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParams p) {
   using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, ALIGNED>;
+  using Fast = FastLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
+  static_assert(!WANT_LA || GENERAL, "the column average uses the general epilogue");
   extern __shared__ __align__(16) unsigned char smem[];
+  float* s_addend = reinterpret_cast<float*>(smem + Tile::LDS_BYTES);  // [2][256]
 
   // XCD-aware item id: workgroup ids that land on one XCD get consecutive items.
   const int xcd = blockIdx.x & 7;
@@ -60,15 +104,27 @@ __global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
 
   typename Tile::CLoader cl;
   typename Tile::ELoader el;
+  typename Fast::CLoader fcl;
+  typename Fast::ELoader fel;
+  if (FAST) {
 #pragma unroll
-  for (int q = 0; q < Tile::ELoader::NQ; ++q) {
-    const int64_t i = t0 + (tid >> 3) + q * Tile::ELoader::ROWSTEP;
-    const uint16_t* ptr = nullptr;
-    if (i < p.b) {
+    for (int q = 0; q < Fast::ELoader::NQ; ++q) {
+      int64_t i = t0 + (tid >> 2) + q * Fast::ELoader::ROWSTEP;
+      i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
       const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
-      ptr = p.e + row * p.stride_e;
+      fel.ptr[q] = p.e + row * p.stride_e + (tid & 3) * 8;
     }
-    el.ptr[q] = ptr;
+  } else {
+#pragma unroll
+    for (int q = 0; q < Tile::ELoader::NQ; ++q) {
+      const int64_t i = t0 + (tid >> 3) + q * Tile::ELoader::ROWSTEP;
+      const uint16_t* ptr = nullptr;
+      if (i < p.b) {
+        const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
+        ptr = p.e + row * p.stride_e;
+      }
+      el.ptr[q] = ptr;
+    }
   }
 
   float m2[kFwdWT], sum[kFwdWT];
@@ -78,41 +134,77 @@ __global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
     sum[ti] = 0.0f;
   }
 
-  // rows of this lane that exist (needed for the optional column average only)
-  float tok_ok[kFwdWT];
-#pragma unroll
-  for (int ti = 0; ti < kFwdWT; ++ti)
-    tok_ok[ti] = (t0 + wt * 128 + ti * 32 + l32 < p.b) ? 1.0f : 0.0f;
-
   for (int vt = vt_begin; vt < vt_end; ++vt) {
     const int64_t v0 = static_cast<int64_t>(vt) * Tile::TILE_V;
+    float* addend = s_addend + (vt & 1) * kFwdTile;
+    if (GENERAL) {
+      // Written before the main loop, whose barriers publish it; the other buffer may still be read
+      // by a wave that is finishing the previous tile.
+      if (tid < kFwdTile) {
+        const int64_t vg = v0 + tid;
+        float a = -INFINITY;
+        if (vg < p.v) a = (p.bias != nullptr) ? Elem<T>::to_float(p.bias[vg]) : 0.0f;
+        addend[tid] = a;
+      }
+    }
+    f32x16 acc[kFwdWV][kFwdWT];
+    if (FAST) {
 #pragma unroll
-    for (int q = 0; q < Tile::CLoader::NQ; ++q) {
-      const int64_t vr = v0 + (tid >> 3) + q * Tile::CLoader::ROWSTEP;
-      cl.ptr[q] = (vr < p.v) ? p.c + vr * p.stride_cv : nullptr;
+      for (int q = 0; q < Fast::CLoader::NQ; ++q) {
+        int64_t vr = v0 + (tid >> 2) + q * Fast::CLoader::ROWSTEP;
+        vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked below
+        fcl.ptr[q] = p.c + vr * p.stride_cv + (tid & 3) * 8;
+      }
+      Fast::run(acc, fcl, fel, smem, static_cast<int>(p.d));
+    } else {
+#pragma unroll
+      for (int q = 0; q < Tile::CLoader::NQ; ++q) {
+        const int64_t vr = v0 + (tid >> 3) + q * Tile::CLoader::ROWSTEP;
+        cl.ptr[q] = (vr < p.v) ? p.c + vr * p.stride_cv : nullptr;
+      }
+      Tile::run(acc, cl, el, smem, static_cast<int>(p.d), p.stride_cd);
     }
 
-    f32x16 acc[kFwdWV][kFwdWT];
-    Tile::run(acc, cl, el, smem, static_cast<int>(p.d), p.stride_cd);
-
-    // ---- epilogue: bias, soft-cap, mask, online max / sum-exp ---------------------------------
-    const int64_t vw0 = v0 + wv * 128;  // first class of this wave
-    const bool ragged = (vw0 + 128 > p.v);
+    // ---- epilogue: (bias, mask,) soft-cap, online max / sum-exp ---------------------------------
+    // One 32-row column block at a time, so that only 64 soft-capped logits are live at once.
+    const int64_t vw0 = v0 + wv * (32 * kFwdWV);  // first class of this wave
+    const float* wave_addend = addend + wv * (32 * kFwdWV);
+    float colsum[WANT_LA ? kFwdWV * 16 : 1];
+    if (WANT_LA) {
 #pragma unroll
-    for (int vi = 0; vi < kFwdWV; ++vi) {
+      for (int j = 0; j < kFwdWV * 16; ++j) colsum[j] = 0.0f;
+    }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t vg = vw0 + vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        float bias = 0.0f;
-        if (p.bias != nullptr && vg < p.v) bias = Elem<T>::to_float(p.bias[vg]);
-        const bool dead = ragged && (vg >= p.v);
+    for (int ti = 0; ti < kFwdWT; ++ti) {
+      __builtin_amdgcn_sched_barrier(0);  // keep each column block's register use to itself
+      float s2[kFwdWV][16];
+      const float tm = column_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, half, s2);
+      if (WANT_LA) {
+        const float ok = (t0 + wt * (32 * kFwdWT) + ti * 32 + l32 < p.b) ? 1.0f : 0.0f;
 #pragma unroll
-        for (int ti = 0; ti < kFwdWT; ++ti) {
-          float th;
-          float s2 = softcap_log2(p.sc, acc[vi][ti][r] + bias, th);
-          acc[vi][ti][r] = dead ? -INFINITY : s2;
-        }
+        for (int vi = 0; vi < kFwdWV; ++vi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) colsum[vi * 16 + r] += (s2[vi][r] == -INFINITY) ? 0.0f : s2[vi][r] * ok;
       }
+
+      if (p.tile_max != nullptr) {
+        // max over the 32 rows x 128 classes of this (wave, ti) cell
+        const float cell = wave_max(tm);
+        const int64_t srow = (t0 + wt * (32 * kFwdWT) + ti * 32) / CCE_STAT_ROWS;
+        const int64_t scol = vw0 / CCE_STAT_COLS;
+        if (lane == 0 && (t0 + wt * (32 * kFwdWT) + ti * 32) < p.b && vw0 < p.v)
+          p.tile_max[srow * p.stat_cols + scol] = cell * kLn2;
+      }
+
+      const float mn = fmaxf(m2[ti], tm);
+      const float ms = (mn == -INFINITY) ? 0.0f : mn;
+      float part = 0.0f;
+#pragma unroll
+      for (int vi = 0; vi < kFwdWV; ++vi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part += __builtin_amdgcn_exp2f(s2[vi][r] - ms);
+      sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + part;
+      m2[ti] = mn;
     }
 
     if (WANT_LA) {
@@ -123,45 +215,12 @@ __global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t vg = vw0 + vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          float colsum = 0.0f;
+          float cs = colsum[vi * 16 + r];
 #pragma unroll
-          for (int ti = 0; ti < kFwdWT; ++ti) {
-            float x = acc[vi][ti][r];
-            colsum += (vg < p.v) ? x * tok_ok[ti] : 0.0f;
-          }
-#pragma unroll
-          for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
-          if (l32 == 0 && vg < p.v) unsafeAtomicAdd(p.logit_avg + vg, colsum * inv_b);
+          for (int off = 16; off >= 1; off >>= 1) cs += __shfl_xor(cs, off, 64);
+          if (l32 == 0 && vg < p.v) unsafeAtomicAdd(p.logit_avg + vg, cs * inv_b);
         }
       }
-    }
-
-#pragma unroll
-    for (int ti = 0; ti < kFwdWT; ++ti) {
-      float tm = -INFINITY;
-#pragma unroll
-      for (int vi = 0; vi < kFwdWV; ++vi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) tm = fmaxf(tm, acc[vi][ti][r]);
-
-      if (p.tile_max != nullptr) {
-        // max over the 32 rows x 128 classes of this (wave, ti) cell
-        const float cell = wave_max(tm);
-        const int64_t srow = (t0 + wt * 128 + ti * 32) / CCE_STAT_ROWS;
-        const int64_t scol = vw0 / CCE_STAT_COLS;
-        if (lane == 0 && (t0 + wt * 128 + ti * 32) < p.b && vw0 < p.v)
-          p.tile_max[srow * p.stat_cols + scol] = cell * kLn2;
-      }
-
-      const float mn = fmaxf(m2[ti], tm);
-      const float ms = (mn == -INFINITY) ? 0.0f : mn;
-      float part = 0.0f;
-#pragma unroll
-      for (int vi = 0; vi < kFwdWV; ++vi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) part += __builtin_amdgcn_exp2f(acc[vi][ti][r] - ms);
-      sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + part;
-      m2[ti] = mn;
     }
   }
 
@@ -188,7 +247,7 @@ __global__ __launch_bounds__(256, 1) void lse_forward_kernel(LseFwdParams p) {
       const float mn = fmaxf(m2[ti], o.x);
       const float ms = (mn == -INFINITY) ? 0.0f : mn;
       const float s = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + o.y * __builtin_amdgcn_exp2f(o.x - ms);
-      const int64_t i = t0 + wt * 128 + ti * 32 + l32;
+      const int64_t i = t0 + wt * (32 * kFwdWT) + ti * 32 + l32;
       if (i < p.b) p.partial[static_cast<int64_t>(split) * p.b + i] = make_float2(mn, s);
     }
   }
@@ -236,21 +295,27 @@ static int choose_nsplit(int nrb, int nvt) {
 template <typename T>
 static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipStream_t stream) {
   using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, true>;
-  const int lds = Tile::LDS_BYTES;
+  using Fast = FastLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
+  static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
+  const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
+  const bool fast = aligned && (p.d % kFastBK == 0) && !want_la;
+  const bool general = want_la || (p.bias != nullptr) || (p.v % Tile::TILE_V != 0);
   const int grid = p.items_per_xcd * 8;
   hipError_t err;
-#define CCE_LAUNCH_FWD(AL, LA)                                                                    \
+#define CCE_LAUNCH_FWD(FA, AL, GE, LA)                                                            \
   do {                                                                                            \
-    auto kern = lse_forward_kernel<T, AL, LA>;                                                    \
+    auto kern = lse_forward_kernel<T, FA, AL, GE, LA>;                                            \
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
     if (err != hipSuccess) return status_from_hip(err);                                           \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, p);                              \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                           \
   } while (0)
-  if (aligned) {
-    if (want_la) CCE_LAUNCH_FWD(true, true); else CCE_LAUNCH_FWD(true, false);
+  if (fast) {
+    if (general) CCE_LAUNCH_FWD(true, true, true, false); else CCE_LAUNCH_FWD(true, true, false, false);
+  } else if (aligned) {
+    if (want_la) CCE_LAUNCH_FWD(false, true, true, true); else CCE_LAUNCH_FWD(false, true, true, false);
   } else {
-    if (want_la) CCE_LAUNCH_FWD(false, true); else CCE_LAUNCH_FWD(false, false);
+    if (want_la) CCE_LAUNCH_FWD(false, false, true, true); else CCE_LAUNCH_FWD(false, false, true, false);
   }
 #undef CCE_LAUNCH_FWD
   return status_from_hip(hipGetLastError());
