@@ -1,0 +1,73 @@
+"""The C-ABI library loads and exports every symbol include/cce_hip.h declares; the host-only
+queries answer without a GPU.  No compute entry point is called here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "cce_hip.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cce_[a-z_0-9]+)\s*\(", text)))
+
+
+def _lib():
+    from cut_cross_entropy import _hip
+
+    if not os.path.exists(_hip.lib_path()):
+        pytest.fail(f"{_hip.lib_path()} is missing: run __graft_entry__.build() first")
+    return _hip.load()
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    for want in ("cce_version", "cce_error_string", "cce_tile_stat_elems", "cce_lse_forward_workspace_bytes",
+                 "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward"):
+        assert want in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib()
+    for name in _declared_functions():
+        assert hasattr(lib, name), f"libcce_hip.so does not export {name}"
+
+
+def test_binding_covers_every_declared_symbol():
+    from cut_cross_entropy import _hip
+
+    assert sorted(_hip._SIGNATURES) == _declared_functions()
+
+
+def test_host_only_queries():
+    lib = _lib()
+    from cut_cross_entropy import _hip
+
+    assert lib.cce_version() == _hip.ABI_VERSION
+    assert lib.cce_error_string(0) == b"success"
+    assert b"workspace" in lib.cce_error_string(10003)
+    # ceil(8192 / 32) * ceil(256000 / 128)
+    assert lib.cce_tile_stat_elems(8192, 256000) == 256 * 2000
+    assert lib.cce_tile_stat_elems(33, 129) == 2 * 2
+    assert lib.cce_tile_stat_elems(0, 100) == 0
+    ws = lib.cce_lse_forward_workspace_bytes(8192, 256000, 2304)
+    assert ws > 0 and ws % 8 == 0 and ws <= 16 * 2**20
+    # one bit per 32 x 32 sub-tile, rows padded to 32-bit words
+    assert lib.cce_backward_workspace_bytes(8192, 256000, 2304) == 256 * 250 * 4
+    assert lib.cce_backward_workspace_bytes(0, 5, 5) == 0
+
+
+def test_header_constants_match_binding():
+    from cut_cross_entropy import _hip
+
+    text = open(HEADER).read()
+    assert int(re.search(r"#define CCE_STAT_ROWS (\d+)", text).group(1)) == _hip.STAT_ROWS
+    assert int(re.search(r"#define CCE_STAT_COLS (\d+)", text).group(1)) == _hip.STAT_COLS
+    assert int(re.search(r"#define CCE_NUM_COUNTERS (\d+)", text).group(1)) == _hip.NUM_COUNTERS
+    assert int(re.search(r"#define CCE_DTYPE_BF16 (\d+)", text).group(1)) == 0
+    assert int(re.search(r"#define CCE_DTYPE_F16 (\d+)", text).group(1)) == 1
