@@ -343,9 +343,10 @@ struct FastLogitTile {
   }
 
   // Issue order of one stage: the memory instructions are spread evenly between the MFMAs, so that
-  // the matrix pipe never waits for a burst of loads to issue.  First half: the global loads and the
-  // fragment reads of step 1; second half: the LDS stores and the fragment reads of the next stage.
-  template <int FIRST_MASK>
+  // the matrix pipe never waits for a burst of loads to issue.  First half: the global loads, then
+  // the fragment reads of step 1; second half: the LDS stores, then the fragment reads of the next
+  // stage (measured: this order beats fragment reads first).
+  template <int OTHER_MASK>
   static __device__ __forceinline__ void interleave_half() {
     constexpr int kMfma = 0x008, kDsRead = 0x100;
     constexpr int nmem = CLoader::NQ + ELoader::NQ;  // global loads = LDS stores per stage
@@ -357,7 +358,7 @@ struct FastLogitTile {
       __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
 #pragma unroll
       for (int j = i * total / nmma; j < (i + 1) * total / nmma; ++j) {
-        if (j < nmem) __builtin_amdgcn_sched_group_barrier(FIRST_MASK, 1, 0);
+        if (j < nmem) __builtin_amdgcn_sched_group_barrier(OTHER_MASK, 1, 0);
         else __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
       }
     }
@@ -443,6 +444,162 @@ struct FastLogitTile {
       CCE_FAST_STAGE(nk - 1, rc1, re1, rc0, re0);
     }
 #undef CCE_FAST_STAGE
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Logit tile with direct global -> LDS loads (gfx950 `global_load_lds_dwordx4`): the data never
+// passes through registers and no wave spends issue slots on LDS stores.
+//
+// Stage = 64 reduction columns = 128-byte rows, so that every row segment is one full cache line
+// (measured: the L2 -> LDS path delivers ~16 TB/s with 128-byte segments, ~12 TB/s with 64-byte
+// ones, and that path is as scarce as the MFMA time at this tile size).  One load writes 64 lanes x
+// 16 bytes = 1 KB of contiguous LDS = 8 rows; lane l lands in row (l >> 3), chunk slot (l & 7) of its
+// block and fetches global chunk slot ^ ((row >> 1) & 7), the XOR swizzle the fragment reads undo
+// (16 consecutive rows x one chunk then cover all 64 banks).  Block b of a stage (b = q * NW + wave)
+// holds rows [8 b, 8 b + 8): class rows first, then token rows.
+//
+// The loads are inline assembly (the compiler would otherwise wait for every outstanding load
+// before the next LDS read) and completion is tracked by hand: two LDS stages, one barrier per stage
+// placed before the last of the four 16-column steps.  At that barrier every wave has read its last
+// fragments of stage s, so the loads of stage s + 2 are issued into that LDS stage right there (a
+// full stage of MFMAs before they are awaited), and the first fragments of stage s + 1 are read
+// under the MFMAs of the last step.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_dma16(const void* gptr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr)
+               : "memory", "m0");
+}
+
+constexpr int kDmaBK = 64;
+constexpr int kDmaRowBytes = 128;
+
+template <typename T, int WV, int WT, int NWV, int NWT>
+struct DmaLogitTile {
+  static constexpr int TILE_V = 32 * WV * NWV;
+  static constexpr int TILE_T = 32 * WT * NWT;
+  static constexpr int NW = NWV * NWT;
+  static constexpr int NT = 64 * NW;
+  static constexpr int STAGE_BYTES = (TILE_V + TILE_T) * kDmaRowBytes;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int NQC = TILE_V / 8 / NW;  // loads per wave and stage that fetch class rows
+  static constexpr int NQE = TILE_T / 8 / NW;  // ... token rows
+  static constexpr int NQ = NQC + NQE;
+  static constexpr int NSTEP = kDmaBK / 16;
+  static_assert(TILE_V % (8 * NW) == 0 && TILE_T % (8 * NW) == 0, "blocks must divide over the waves");
+  static_assert(NW % 2 == 0, "the swizzle of a lane must not depend on q");
+  using vec8 = typename Elem<T>::vec8;
+
+  // Tile row (class or token index inside the tile) that this lane fetches with load q.
+  static __device__ __forceinline__ int row_of(int q, int wave, int lane) {
+    const int q2 = (q < NQC) ? q : q - NQC;
+    return 8 * (q2 * NW + wave) + (lane >> 3);
+  }
+  // Element offset inside a 64-column stage of the chunk this lane fetches.
+  static __device__ __forceinline__ int chunk_elems(int wave, int lane) {
+    const int sw = (4 * (wave & 1) + (lane >> 4)) & 7;  // (row >> 1) & 7 for row = 8 * block + (lane >> 3)
+    return ((lane & 7) ^ sw) * 8;
+  }
+
+  struct Frags {
+    vec8 a[WV];
+    vec8 b[WT];
+  };
+
+  static __device__ __forceinline__ Frags read_frags(const unsigned char* lds, int stage_off, int kk, int coff0,
+                                                     int eoff0, int sw, int half) {
+    Frags f;
+    const int chunk = (((kk * 2 + half) ^ sw) << 4);
+    const unsigned char* cb = lds + stage_off + coff0 + chunk;
+    const unsigned char* eb = lds + stage_off + eoff0 + chunk;
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+      f.a[vi] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(cb + vi * 32 * kDmaRowBytes));
+#pragma unroll
+    for (int ti = 0; ti < WT; ++ti)
+      f.b[ti] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(eb + ti * 32 * kDmaRowBytes));
+    return f;
+  }
+
+  static __device__ __forceinline__ void mma(f32x16 (&acc)[WV][WT], const Frags& f) {
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
+  }
+
+  // Issue the NQ loads of one stage (columns [k0, k0 + 64)) into LDS stage `stage_off`.
+  static __device__ __forceinline__ void issue(const uint16_t* const (&ptr)[NQ], int k0, unsigned lds_base,
+                                               int stage_off, int wave) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int blk = (q < NQC) ? (q * NW + wave) : (TILE_V / 8 + (q - NQC) * NW + wave);
+      lds_dma16(ptr[q] + k0, lds_base + stage_off + blk * 1024);
+    }
+  }
+
+  // D must be a multiple of 64.
+  static __device__ __forceinline__ void run(f32x16 (&acc)[WV][WT], const uint16_t* const (&ptr)[NQ],
+                                             unsigned char* lds, int D) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wv = wave / NWT;
+    const int wt = wave % NWT;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int sw = (l32 >> 1) & 7;
+    const int coff0 = (wv * WV * 32 + l32) * kDmaRowBytes;
+    const int eoff0 = (TILE_V + wt * WT * 32 + l32) * kDmaRowBytes;
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[vi][ti][r] = 0.0f;
+
+    const int nk = D / kDmaBK;
+    const int last = (nk - 1) * kDmaBK;
+    issue(ptr, 0, lds_base, 0, wave);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    issue(ptr, min(kDmaBK, last), lds_base, STAGE_BYTES, wave);
+    Frags fa = read_frags(lds, 0, 0, coff0, eoff0, sw, half);
+    Frags fb;
+
+    // The scheduling fences pin "reads of the next step first, then this step's MFMAs": left alone,
+    // the compiler sinks every LDS read next to its use and the LDS latency is exposed.
+#pragma unroll 1
+    for (int s = 0; s < nk; ++s) {
+      const int cur = (s & 1) * STAGE_BYTES;
+      const int nxt = STAGE_BYTES - cur;
+      fb = read_frags(lds, cur, 1, coff0, eoff0, sw, half);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(acc, fa);  // step 0
+      __builtin_amdgcn_sched_barrier(0);
+      fa = read_frags(lds, cur, 2, coff0, eoff0, sw, half);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(acc, fb);  // step 1
+      __builtin_amdgcn_sched_barrier(0);
+      fb = read_frags(lds, cur, 3, coff0, eoff0, sw, half);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(acc, fa);  // step 2
+      __builtin_amdgcn_sched_barrier(0);
+      // Stage s + 1 (issued a full stage ago) has landed for this wave; after the barrier, for every
+      // wave, and every wave holds its last fragments of stage s in registers: that LDS stage is free
+      // and the loads of stage s + 2 go into it.  A prefetch past the end re-reads the last stage
+      // (never consumed), which keeps the loop free of branches.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      issue(ptr, min((s + 2) * kDmaBK, last), lds_base, cur, wave);
+      fa = read_frags(lds, nxt, 0, coff0, eoff0, sw, half);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(acc, fb);  // step 3
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch
+    __syncthreads();  // every wave is done with the LDS (the last prefetch was awaited above)
   }
 };
 

@@ -70,14 +70,14 @@ __device__ __forceinline__ float column_block_logits(const Softcap& sc, const f3
 }
 
 // Kernel variants:
-//   FAST     rows 16-byte aligned, unit column stride, D % 32 == 0: software-pipelined main loop
+//   FAST     rows 16-byte aligned, unit column stride, D % 64 == 0: direct-to-LDS pipelined main loop
 //   ALIGNED  (generic main loop only) 16-byte vector loads are legal
 //   GENERAL  a bias is present or V is not a multiple of the tile: per-class addend / mask from LDS
 //   WANT_LA  also accumulate the column average of the logits (needs GENERAL)
 template <typename T, bool FAST, bool ALIGNED, bool GENERAL, bool WANT_LA>
 __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParams p) {
   using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, ALIGNED>;
-  using Fast = FastLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
+  using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(!WANT_LA || GENERAL, "the column average uses the general epilogue");
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_addend = reinterpret_cast<float*>(smem + Tile::LDS_BYTES);  // [2][256]
@@ -104,15 +104,14 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
 
   typename Tile::CLoader cl;
   typename Tile::ELoader el;
-  typename Fast::CLoader fcl;
-  typename Fast::ELoader fel;
+  const uint16_t* fptr[Fast::NQ];  // FAST: per-lane source of each direct-to-LDS load
   if (FAST) {
 #pragma unroll
-    for (int q = 0; q < Fast::ELoader::NQ; ++q) {
-      int64_t i = t0 + (tid >> 2) + q * Fast::ELoader::ROWSTEP;
+    for (int q = Fast::NQC; q < Fast::NQ; ++q) {
+      int64_t i = t0 + Fast::row_of(q, wave, lane);
       i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
       const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
-      fel.ptr[q] = p.e + row * p.stride_e + (tid & 3) * 8;
+      fptr[q] = p.e + row * p.stride_e + Fast::chunk_elems(wave, lane);
     }
   } else {
 #pragma unroll
@@ -150,12 +149,12 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
     f32x16 acc[kFwdWV][kFwdWT];
     if (FAST) {
 #pragma unroll
-      for (int q = 0; q < Fast::CLoader::NQ; ++q) {
-        int64_t vr = v0 + (tid >> 2) + q * Fast::CLoader::ROWSTEP;
+      for (int q = 0; q < Fast::NQC; ++q) {
+        int64_t vr = v0 + Fast::row_of(q, wave, lane);
         vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked below
-        fcl.ptr[q] = p.c + vr * p.stride_cv + (tid & 3) * 8;
+        fptr[q] = p.c + vr * p.stride_cv + Fast::chunk_elems(wave, lane);
       }
-      Fast::run(acc, fcl, fel, smem, static_cast<int>(p.d));
+      Fast::run(acc, fptr, smem, static_cast<int>(p.d));
     } else {
 #pragma unroll
       for (int q = 0; q < Tile::CLoader::NQ; ++q) {
@@ -295,10 +294,10 @@ static int choose_nsplit(int nrb, int nvt) {
 template <typename T>
 static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipStream_t stream) {
   using Tile = LogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT, true>;
-  using Fast = FastLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
+  using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
   const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
-  const bool fast = aligned && (p.d % kFastBK == 0) && !want_la;
+  const bool fast = aligned && (p.d % kDmaBK == 0) && !want_la;
   const bool general = want_la || (p.bias != nullptr) || (p.v % Tile::TILE_V != 0);
   const int grid = p.items_per_xcd * 8;
   hipError_t err;
