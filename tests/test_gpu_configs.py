@@ -1,0 +1,350 @@
+"""Parity at the benchmark configurations (scaled where the dense oracle would not fit in seconds,
+full size for the headline shape), plus the properties that only show at scale: gradient
+filtering with the no-recompute shortcut, determinism, class permutation, vocabulary shards."""
+
+import math
+
+import pytest
+import torch
+
+from _util import IGNORE_INDEX
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _gen(N, D, V, seed=0, e_std=1.0, c_std=0.02, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    e = (torch.randn((N, D), generator=g) * e_std).to(dtype)
+    c = (torch.randn((V, D), generator=g) * c_std).to(dtype)
+    t = torch.randint(0, V, (N,), generator=g)
+    return e, c, t, g
+
+
+def _oracle_on_gpu(e, c, t, valids, d_out, d_lse, softcap, shift=0, bias=None, filter_eps=None):
+    """Dense fp32 oracle evaluated with torch on the GPU, row-chunked: LSE and gradients.
+
+    With ``filter_eps`` the gradient filter is restated exactly as specified: the plane of
+    (valid row, class) is cut into 32 x 32 sub-tiles and a sub-tile whose every |p - onehot| is
+    below ``filter_eps`` contributes nothing (reference rule, cce_backward.py:211-216, at this
+    build's tile size).  The inputs of these tests keep |p - onehot| far from the threshold, so
+    the kept set does not depend on rounding."""
+    from oracle import dense_lce
+
+    N, D = e.shape
+    V = c.shape[0]
+    rows = torch.arange(N, device=e.device) if valids is None else valids.long()
+    lse = torch.cat([dense_lce.dense_lse(e[r], c, bias, softcap, torch.float32) for r in rows.split(2048)])
+    if filter_eps is None:
+        de, dc, db = dense_lce.dense_grads(e, c, t, valids, d_out, d_lse, bias, softcap, shift, torch.float32, chunk=1024)
+        return lse, de, dc, db
+    assert bias is None and d_lse is None
+    cc = c.float()
+    de = torch.zeros((N, D), dtype=torch.float32, device=e.device)
+    dc = torch.zeros((V, D), dtype=torch.float32, device=e.device)
+    Vp = (V + 31) // 32 * 32
+    for s0 in range(0, rows.numel(), 1024):
+        r = rows[s0 : s0 + 1024]
+        ee = e[r].float()
+        z = ee @ cc.T
+        sl = dense_lce.softcapping(z, softcap) if softcap is not None else z
+        p = torch.exp(sl - lse[s0 : s0 + 1024, None])
+        tt = t[r + shift]
+        y = torch.zeros_like(p)
+        y.scatter_(1, tt.view(-1, 1), 1.0)
+        f = (p - y).abs()
+        n = r.numel()
+        npad = (n + 31) // 32 * 32
+        fp = torch.zeros((npad, Vp), device=e.device)
+        fp[:n, :V] = f
+        keep = fp.view(npad // 32, 32, Vp // 32, 32).amax(dim=(1, 3)) >= filter_eps
+        keep = keep[:, None, :, None].expand(-1, 32, -1, 32).reshape(npad, Vp)[:n, :V]
+        g = d_out[r + shift].view(-1, 1) if d_out.numel() > 1 else d_out.reshape(())
+        dz = (p - y) * g
+        if softcap is not None:
+            dz = dz * (1 - (sl / softcap) ** 2)
+        dz = dz * keep
+        de.index_add_(0, r, dz @ cc)
+        dc += dz.T @ ee
+    return lse, de, dc, None
+
+
+def _rel_err(got, want):
+    scale = want.abs().max().item()
+    return (got.float() - want.float()).abs().max().item() / max(scale, 1e-30)
+
+
+def test_config1_small_reference_run():
+    """N=4096, D=1024, V=32000, 5 % ignored, mean, seed 0.  Loss against the fp32 oracle on the CPU;
+    gradients against the oracle with the filter rule applied (default impl="cce" filters)."""
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import _build_flat_valids
+    from oracle import dense_lce
+
+    N, D, V = 4096, 1024, 32000
+    e, c, t, g = _gen(N, D, V, seed=0)
+    t[torch.randperm(N, generator=g)[: int(0.05 * N)]] = IGNORE_INDEX
+    want, _ = dense_lce.dense_linear_cross_entropy(e.float(), c.float(), t)
+
+    ed = e.to(DEV).requires_grad_(True)
+    cd = c.to(DEV).requires_grad_(True)
+    td = t.to(DEV)
+    loss = linear_cross_entropy(ed, cd, td, impl="cce")
+    loss.backward()
+    assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+    valids = _build_flat_valids(td, IGNORE_INDEX, 0)
+    d_out = torch.full((N,), 1.0 / valids.numel(), device=DEV)
+    _, de, dc, _ = _oracle_on_gpu(e.to(DEV), c.to(DEV), td.clamp_min(0), valids, d_out, None, None,
+                                  filter_eps=2.0**-12)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+    ign = t == IGNORE_INDEX
+    assert (ed.grad.cpu()[ign] == 0).all()  # bit-exact masking
+    # and the unfiltered preset against the unfiltered oracle
+    ed.grad = cd.grad = None
+    linear_cross_entropy(ed, cd, td, impl="cce_exact").backward()
+    _, de, dc, _ = _oracle_on_gpu(e.to(DEV), c.to(DEV), td.clamp_min(0), valids, d_out, None, None)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+
+
+def test_config2_full_size_forward_and_backward():
+    """The headline shape at full size against the dense fp32 oracle run with torch on the GPU:
+    loss / LSE within 1e-3 relative, dE / dC within 1e-2 of the gradient scale with gradient
+    filtering on, loss-path memory under 16 MB, and most of the plane skipped unseen."""
+    from cut_cross_entropy import cce as cce_mod
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, D, V, softcap = 8192, 2304, 256000, 30.0
+    g = torch.Generator(device=DEV).manual_seed(0)
+    e = torch.randn((N, D), generator=g, device=DEV).to(torch.bfloat16)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (N,), generator=g, device=DEV)
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+
+    counters = torch.zeros(4, dtype=torch.int64, device=DEV)
+    cce_mod.set_tile_counters(counters)
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    loss, lse = linear_cross_entropy(ed, cd, t, softcap=softcap, impl="cce", return_lse=True)
+    loss.backward()
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - base
+    cce_mod.set_tile_counters(None)
+    extra_mb = (peak - ed.grad.numel() * 2 - cd.grad.numel() * 2) / 2**20
+    assert extra_mb <= 16.0, extra_mb
+
+    d_out = torch.full((N,), 1.0 / N, device=DEV)
+    want_lse, de, dc, _ = _oracle_on_gpu(e, c, t, None, d_out, None, softcap, filter_eps=2.0**-12)
+    assert torch.allclose(lse, want_lse, rtol=1e-3, atol=1e-3)
+    from oracle import dense_lce
+
+    want_loss = (want_lse + dense_lce.dense_indexed_neg_dot(e, c, t, None, softcap, torch.float32)).mean()
+    assert abs(loss.item() - want_loss.item()) <= 1e-3 * abs(want_loss.item())
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+    total, recomputed, with_de, with_dc = counters.tolist()
+    assert total == (N // 32) * (V // 32)
+    assert recomputed / total < 0.05 and with_de / total < 0.02 and with_dc == with_de
+
+
+@pytest.mark.parametrize("filter_eps", ["auto", None])
+def test_config2_scaled_filter_vs_exact(filter_eps):
+    """Near-uniform soft-max: with filtering only the target sub-tiles survive, and the result stays
+    within the filter's error bound of the unfiltered one."""
+    from cut_cross_entropy import cce as cce_mod
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, D, V = 1024, 2304, 32000
+    e, c, t, _ = _gen(N, D, V, seed=3, c_std=0.01)  # logit std 0.48: every non-target p is well below eps
+    e, c, t = e.to(DEV), c.to(DEV), t.to(DEV)
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    counters = torch.zeros(4, dtype=torch.int64, device=DEV)
+    cce_mod.set_tile_counters(counters)
+    loss = linear_cross_entropy(ed, cd, t, softcap=30.0, impl="cce", filter_eps=filter_eps, reduction="sum")
+    loss.backward()
+    torch.cuda.synchronize()
+    cce_mod.set_tile_counters(None)
+    d_out = torch.ones((N,), device=DEV)
+    _, de, dc, _ = _oracle_on_gpu(e, c, t, None, d_out, None, 30.0,
+                                  filter_eps=None if filter_eps is None else 2.0**-12)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+    total, recomputed, with_de, with_dc = counters.tolist()
+    if filter_eps is None:
+        assert recomputed == total == with_de == with_dc
+    else:
+        # a sub-tile survives iff it holds a target (every other |p| is far below eps here)
+        want = len({(i // 32, int(tt) // 32) for i, tt in enumerate(t.tolist())})
+        # (plus the few sub-tiles where an extreme logit lifts one p above eps)
+        assert want <= with_de <= 1.25 * want and with_dc == with_de
+        assert recomputed < 0.2 * total
+
+
+def test_config3_scaled_shift_and_trailing_ignored():
+    """Llama-shaped call pattern: [batch, T] with shift=1 and the tail of every row ignored."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    Bt, T, D, V = 4, 512, 1024, 16384
+    e, c, t, _ = _gen(Bt * T, D, V, seed=4)
+    t = t.view(Bt, T).clone()
+    t[:, -32:] = IGNORE_INDEX
+    e3 = e.view(Bt, T, D)
+    eo = e3.float().requires_grad_(True)
+    co = c.float().requires_grad_(True)
+    want, _ = dense_lce.dense_linear_cross_entropy(eo, co, t, shift=1)
+    want.backward()
+    ed = e3.to(DEV).requires_grad_(True)
+    cd = c.to(DEV).requires_grad_(True)
+    loss = linear_cross_entropy(ed, cd, t.to(DEV), shift=1, impl="cce")
+    loss.backward()
+    assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+    assert _rel_err(ed.grad.cpu(), eo.grad) <= 1e-2
+    assert _rel_err(cd.grad.cpu(), co.grad) <= 1e-2
+    # rows whose shifted target is ignored (and the last row of every sequence) get exactly zero
+    dead = torch.ones(Bt, T, dtype=torch.bool)
+    dead[:, : T - 1] = t[:, 1:] == IGNORE_INDEX
+    assert (ed.grad.cpu()[dead] == 0).all()
+
+
+def test_config4_scaled_kahan_full_zloss_none():
+    """Zipf labels, impl=cce_kahan_full_c_full_e (no filtering, fp32 accumulation), z-loss with
+    weight 1e-4, reduction none: per-token loss and gradients."""
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import compute_z_loss
+    from oracle import dense_lce
+
+    N, D, V, w = 1024, 2048, 16000, 1e-4
+    e, c, _, g = _gen(N, D, V, seed=5)
+    ranks = torch.arange(1, V + 1, dtype=torch.float64)
+    cdf = torch.cumsum(ranks.pow(-1.1), 0)
+    cdf /= cdf[-1].clone()
+    t = torch.searchsorted(cdf, torch.rand(N, generator=g, dtype=torch.float64)).clamp_max(V - 1)
+    eo = e.float().requires_grad_(True)
+    co = c.float().requires_grad_(True)
+    want, want_lse = dense_lce.dense_linear_cross_entropy(eo, co, t, reduction="none", return_lse=True)
+    (want.mean() + w * dense_lce.compute_z_loss(want_lse, t)).backward()
+    ed = e.to(DEV).requires_grad_(True)
+    cd = c.to(DEV).requires_grad_(True)
+    td = t.to(DEV)
+    loss, lse = linear_cross_entropy(ed, cd, td, impl="cce_kahan_full_c_full_e", reduction="none", return_lse=True)
+    (loss.mean() + w * compute_z_loss(lse, td)).backward()
+    assert torch.allclose(loss.cpu(), want.detach(), rtol=1e-3, atol=1e-3)
+    assert torch.allclose(lse.cpu(), want_lse.detach(), rtol=1e-3, atol=1e-3)
+    assert _rel_err(ed.grad.cpu(), eo.grad) <= 1e-2
+    assert _rel_err(cd.grad.cpu(), co.grad) <= 1e-2
+
+
+def test_config5_scaled_peaked_and_sequential_shards():
+    """Rows aligned with their class vector, then the vocabulary cut into 8 shards that are run one
+    after another on the one GPU and combined on the host (no collective): LSE, loss, dE and dC
+    of the shards recombine to the full-vocabulary result."""
+    from cut_cross_entropy import VocabParallelOptions, linear_cross_entropy
+    from cut_cross_entropy.vocab_parallel import combine_shards, partition_n_into_range, shard_backward, shard_forward
+
+    N, D, V = 2048, 1024, 19008
+    g = torch.Generator().manual_seed(6)
+    c = (torch.randn((V, D), generator=g) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (N,), generator=g)
+    e = (4.0 * c[t].float() + 0.5 * torch.randn((N, D), generator=g)).to(torch.bfloat16)
+    e, c, t = e.to(DEV), c.to(DEV), t.to(DEV)
+
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    full, full_lse = linear_cross_entropy(ed, cd, t, impl="cce_exact", reduction="none", return_lse=True)
+    full.sum().backward()
+
+    corr, lses, bounds = [], [], []
+    for rank in range(8):
+        s, s_end = partition_n_into_range(V, rank, 8)
+        bounds.append((s, s_end))
+        cl, ll = shard_forward(e, c[s:s_end], t, VocabParallelOptions(s, s_end))
+        corr.append(cl)
+        lses.append(ll)
+    nll, lse = combine_shards(corr, lses)
+    assert torch.allclose(lse, full_lse, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(nll, full.detach(), rtol=1e-3, atol=1e-3)
+    # rows whose label another shard holds contribute an exact zero
+    s0, e0 = bounds[0]
+    outside = (t < s0) | (t >= e0)
+    assert (corr[0][outside] == 0).all()
+
+    d_out = torch.ones((N,), device=DEV)
+    de_sum = torch.zeros((N, D), dtype=torch.float32, device=DEV)
+    for (s, s_end) in bounds:
+        de, dc, _ = shard_backward(e, c[s:s_end], t, VocabParallelOptions(s, s_end), lse, d_out)
+        de_sum += de
+        assert _rel_err(dc, cd.grad[s:s_end]) <= 1e-2
+    assert _rel_err(de_sum, ed.grad) <= 1e-2
+
+    # the operator itself with shard bounds: shard-local loss = lse_shard - correct_logit
+    one = linear_cross_entropy(e, c[s0:e0], t, impl="cce_exact", reduction="none",
+                               vocab_parallel_options=VocabParallelOptions(s0, e0))
+    assert torch.allclose(one, lses[0] - corr[0], rtol=1e-5, atol=1e-5)
+
+
+def test_backward_is_deterministic_and_order_invariant():
+    """Two runs give bit-identical gradients, and a class permutation (reference vocab_ordering)
+    changes nothing but the summation order inside a row group."""
+    from cut_cross_entropy.cce_backward import cce_backward_kernel
+    from cut_cross_entropy.cce_lse_forward import cce_lse_forward_kernel
+    from cut_cross_entropy.utils import TensorInfo
+
+    N, D, V = 512, 256, 4000
+    e, c, t, g = _gen(N, D, V, seed=7, c_std=0.05)
+    e, c, t = e.to(DEV), c.to(DEV), t.to(DEV)
+    lse = cce_lse_forward_kernel(e, c)
+    info = TensorInfo(torch.float32, True)
+    do = torch.randn((N,), generator=g).to(DEV)
+
+    def run(order):
+        return cce_backward_kernel(do, None, e, info, c, info, None, None, lse, None, None, None, targets=t,
+                                   vocab_ordering=order, accum_e_fp32=True, accum_c_fp32=True)
+
+    de1, dc1, _ = run(None)
+    de2, dc2, _ = run(None)
+    assert torch.equal(de1, de2) and torch.equal(dc1, dc2)
+    perm = torch.randperm(V, generator=g).to(torch.int32).to(DEV)
+    de3, dc3, _ = run(perm)
+    assert torch.allclose(de1, de3, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(dc1, dc3, rtol=1e-4, atol=1e-5)
+
+
+def test_dlse_only_gradient():
+    """The loss output unused, only the z-loss of the LSE: the gradient arrives through d_lse alone."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    N, D, V = 256, 128, 1000
+    e, c, t, _ = _gen(N, D, V, seed=8, c_std=0.1)
+    eo = e.float().requires_grad_(True)
+    co = c.float().requires_grad_(True)
+    _, lse_o = dense_lce.dense_linear_cross_entropy(eo, co, t, return_lse=True)
+    lse_o.pow(2).mean().backward()
+    ed = e.to(DEV).requires_grad_(True)
+    cd = c.to(DEV).requires_grad_(True)
+    _, lse = linear_cross_entropy(ed, cd, t.to(DEV), impl="cce_exact", return_lse=True)
+    lse.pow(2).mean().backward()
+    assert _rel_err(ed.grad.cpu(), eo.grad) <= 1e-2
+    assert _rel_err(cd.grad.cpu(), co.grad) <= 1e-2
+
+
+def test_strided_classifier_and_lse_kernel_logit_avg():
+    """A classifier that is a column slice of a wider matrix (row stride != D), and the optional
+    column average of the launcher API."""
+    from cut_cross_entropy.cce_lse_forward import cce_lse_forward_kernel
+    from oracle import dense_lce
+
+    N, D, V = 300, 128, 1000
+    e, c_wide, _, _ = _gen(N, D + 64, V, seed=9, c_std=0.1)
+    e = e[:, :D].contiguous().to(DEV)
+    c = c_wide.to(DEV)[:, :D]
+    assert not c.is_contiguous()
+    lse, la = cce_lse_forward_kernel(e, c, softcap=20.0, return_logit_avg=True)
+    logits = dense_lce._dense_logits(e.cpu(), c.cpu(), None, 20.0, torch.float64)
+    assert torch.allclose(lse.cpu().double(), torch.logsumexp(logits, -1), rtol=1e-4, atol=1e-4)
+    assert torch.allclose(la.cpu().double(), logits.mean(0), rtol=2e-2, atol=2e-2)
