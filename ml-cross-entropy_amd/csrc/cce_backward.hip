@@ -4,22 +4,22 @@
 // Global read-modify-write is the slow path of this chip (a few hundred G lane-updates/s), so the
 // two gradients are produced by two ownership kernels whose accumulators never leave registers:
 //
-//   bwd_de_kernel   one workgroup (4 waves) owns 32 valid rows (a "row group") and up to 2304
-//                   columns of dE.  It walks the 128-class cells of the vocabulary that can matter
-//                   for its rows, recomputes logits^T (128 classes x 32 rows) with MFMA, forms
-//                   dz, applies the gradient filter per 32 x 32 sub-tile, and accumulates
-//                   dE^T (D x 32 rows) += C_cell^T . dz^T in fp32 registers (wave w owns the 32-column
-//                   blocks w, w + 4 of every 256).  The rows are written once at the end.  It also records,
-//                   one bit per 32 x 32 sub-tile, which sub-tiles survived the filter.
-//   bwd_dc_kernel   one workgroup owns 32 classes (and up to 2304 columns of dC), walks the row
-//                   groups whose bit is set (all of them when dC is not filtered), recomputes the
-//                   32 x 32 logits, and accumulates dC^T (D x 32 classes) += E_group^T . dz; dBias is
-//                   the row sum of the same dz.  Rows are written once at the end.
+//   dE pass   one workgroup (4 waves) owns 32 valid rows (a "row group") and up to 2304 columns of dE.
+//             It walks the 32-class sub-blocks of the vocabulary that can matter for its rows, four at a
+//             time, recomputes their logits with MFMA, forms dz, applies the gradient filter per
+//             32 x 32 sub-tile, and accumulates dE^T (D x 32 rows) += C_cell^T . dz^T in fp32 registers.
+//             The rows are written once at the end.  It also records, one bit per 32 x 32 sub-tile,
+//             which sub-tiles survived the filter.
+//   dC pass   one workgroup owns 32 classes (and up to 2304 columns of dC), walks the row groups whose
+//             bit is set (all of them when dC is not filtered), four at a time, recomputes the 32 x 32
+//             logits, and accumulates dC^T (D x 32 classes) += E_cell^T . dz; dBias is the row sum of the
+//             same dz.  Rows are written once at the end.
+// Both passes are one kernel template (bwd_owner_kernel) with the roles of E and C swapped.
 //
-// Which cells can matter: the forward pass left, per 32 rows x 128 classes, the largest soft-capped
-// logit.  A cell none of whose rows has its target inside and whose bound
-// exp(cell_max - min_row lse) is below filter_eps has every |p - onehot| below filter_eps, so the
-// filter would drop all four of its sub-tiles: it is skipped without being recomputed.
+// Which sub-blocks can matter: the forward pass left, per 32 rows x 128 classes, the largest
+// soft-capped logit.  If the bound exp(cell_max - min_row lse) of a cell is below filter_eps, every
+// |p| in it is below filter_eps, so only the sub-blocks that hold a target of one of the rows can
+// survive the filter: the others are skipped without being recomputed.
 //
 // The price of ownership is that kept sub-tiles are recomputed once more in the second kernel;
 // with filtering that is a small fraction of the plane.  Results are deterministic.
@@ -223,59 +223,85 @@ __device__ __forceinline__ bool block_epilogue(const BwdParams& p, f32x16& acc, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// dE: workgroup = (row group of 32, slice of D)
+// The ownership kernel, instantiated twice.
+//
+//   IS_DE = true   the workgroup owns 32 valid rows ("own" side = rows of E) and walks class
+//                  sub-blocks of 32 ("other" side = rows of C); it writes dE rows and the survivor
+//                  bits.
+//   IS_DE = false  the workgroup owns 32 classes (own = rows of C) and walks row groups of 32
+//                  (other = rows of E); it writes dC rows and dBias.
+//
+// Four list entries are processed per trip as one "virtual cell" of 128 other-side rows gathered by
+// id (the entries need not be neighbours): wave w recomputes the 32 x 32 logits of entry w against
+// the own rows over all of D, forms dz, and then all four waves accumulate
+//     own_grad^T (D x 32 own) += Other_cell^T (D x 128) . dz (128 x 32 own)
+// with wave w owning the 32-column blocks w and w + 4 of every 256 columns of D.
 // ---------------------------------------------------------------------------------------------
-constexpr int kDeOffC = 0;                          // 64 KB  C stage: 128 classes x 256 columns
-constexpr int kDeOffE = 64 * 1024;                  // 16 KB  E stage: 32 rows x 256 columns
-constexpr int kDeOffDz = 80 * 1024;                 //  8 KB  dz^T [row][class], 256 bytes per row
-constexpr int kDeOffList = 88 * 1024;               // 16 KB  cell list
-constexpr int kDeOffFlag = 104 * 1024;              //  4 KB  cell flags (bytes)
-constexpr int kDeOffBits = 108 * 1024;              //  bit row, then metadata
-constexpr int kDeMaxBitWords = 2048;                //  8 KB  (V <= 2 M classes)
-constexpr int kDeOffMeta = kDeOffBits + kDeMaxBitWords * 4;
-constexpr int kDeLdsBytes = kDeOffMeta + 5 * 128 + 512 + 64;
+constexpr int kOffOther = 0;                      // 64 KB  other-side stage: 128 rows x 256 columns
+constexpr int kOffOwn = 64 * 1024;                // 16 KB  own-side stage: 32 rows x 256 columns
+constexpr int kOffDz = 80 * 1024;                 //  8 KB  dz [own][other], 256 bytes per own row
+constexpr int kOffList = 88 * 1024;               // 16 KB  entry list
+constexpr int kOffFlag = 104 * 1024;              //  1 KB  per-cell sub-block masks (dE)
+constexpr int kOffBits = 105 * 1024;              //  8 KB  survivor-bit row (dE)
+constexpr int kMaxBitWords = 2048;                //        (V <= 2 M classes)
+constexpr int kOffMeta = kOffBits + kMaxBitWords * 4;
+constexpr int kMetaRows = 128;
+constexpr int kBwdLdsBytes = kOffMeta + 5 * kMetaRows * 4 + 32 * 4 + 128 * 4 + 128 * 4 + 64;
+constexpr int kSegCells = 1024;                   // dE: 128-class cells scanned per pass (<= 4096 entries)
 
-template <typename T, bool ALIGNED>
-__global__ __launch_bounds__(kBwdThreads, 1) void bwd_de_kernel(BwdParams p) {
+template <typename T, bool ALIGNED, bool IS_DE>
+__global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sC = smem + kDeOffC;
-  unsigned char* sE = smem + kDeOffE;
-  unsigned char* sDz = smem + kDeOffDz;
-  int* sList = reinterpret_cast<int*>(smem + kDeOffList);
-  unsigned char* sFlag = smem + kDeOffFlag;
-  uint32_t* sBits = reinterpret_cast<uint32_t*>(smem + kDeOffBits);
-  RowMeta meta;
-  meta.row = reinterpret_cast<int*>(smem + kDeOffMeta);
-  meta.tgt = meta.row + 32;
-  meta.lse2 = reinterpret_cast<float*>(meta.tgt + 32);
-  meta.g = meta.lse2 + 32;
-  meta.h = meta.g + 32;
-  int* sCid = reinterpret_cast<int*>(meta.h + 32);  // [128]
-  int* sMisc = sCid + 128;                           // [0] list length, [1] kept-block mask, [2] min lse
+  unsigned char* sOther = smem + kOffOther;
+  unsigned char* sOwn = smem + kOffOwn;
+  unsigned char* sDz = smem + kOffDz;
+  int* sList = reinterpret_cast<int*>(smem + kOffList);
+  unsigned char* sFlag = smem + kOffFlag;
+  uint32_t* sBits = reinterpret_cast<uint32_t*>(smem + kOffBits);
+  RowMeta meta;  // per token row: 32 own rows (dE) or the 128 rows of the current virtual cell (dC)
+  meta.row = reinterpret_cast<int*>(smem + kOffMeta);
+  meta.tgt = meta.row + kMetaRows;
+  meta.lse2 = reinterpret_cast<float*>(meta.tgt + kMetaRows);
+  meta.g = meta.lse2 + kMetaRows;
+  meta.h = meta.g + kMetaRows;
+  int* sOwnCid = reinterpret_cast<int*>(meta.h + kMetaRows);  // [32]  dC: class ids of the own rows
+  int* sCellCid = sOwnCid + 32;                                // [128] dE: class ids of the virtual cell
+  float* sDb = reinterpret_cast<float*>(sCellCid + 128);       // [4][32] dC: per-wave dBias of the own classes
+  int* sMisc = reinterpret_cast<int*>(sDb + 128);               // [0] list length, [1] entry mask, [2] min lse
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int half = lane >> 5;
-  const int tg = blockIdx.x / p.nslices;
+  const int own = blockIdx.x / p.nslices;  // row group (dE) or class group (dC)
   const int slice = blockIdx.x % p.nslices;
   const int d_begin = slice * p.dslice;
   const int d_end = min(static_cast<int>(p.d), d_begin + p.dslice);
   const int nchunks = (d_end - d_begin + kStageCols - 1) / kStageCols;
   const int D = static_cast<int>(p.d);
-  const bool write_de = (p.d_e != nullptr);
+  const bool write_out = IS_DE ? (p.d_e != nullptr) : (p.d_c != nullptr);
 
-  // ---- row metadata, minimum lse of the group ------------------------------------------------
+  // ---- own-side metadata -----------------------------------------------------------------------
   float my_lse = INFINITY;
-  if (tid < 32) my_lse = load_row_meta(p, static_cast<int64_t>(tg) * 32 + tid, tid, meta);
-  if (wave == 0) {
-    const float mn = wave_min(my_lse);
-    if (lane == 0) reinterpret_cast<float*>(sMisc)[2] = mn;
+  if (IS_DE) {
+    if (tid < 32) my_lse = load_row_meta(p, static_cast<int64_t>(own) * 32 + tid, tid, meta);
+    if (wave == 0) {
+      const float mn = wave_min(my_lse);
+      if (lane == 0) reinterpret_cast<float*>(sMisc)[2] = mn;
+    }
+    for (int w = tid; w < p.bit_words; w += kBwdThreads) sBits[w] = 0u;
+  } else if (tid < 32) {
+    const int64_t pos = static_cast<int64_t>(own) * 32 + tid;
+    int cid = -1;
+    if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
+    sOwnCid[tid] = cid;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sDb[w * 32 + tid] = 0.0f;
   }
-  for (int w = tid; w < p.bit_words; w += kBwdThreads) sBits[w] = 0u;
   __syncthreads();
   const float min_lse = reinterpret_cast<float*>(sMisc)[2];
+  const int* own_ids = IS_DE ? meta.row : sOwnCid;
 
   // wave w owns columns [32 w, 32 w + 32) and [128 + 32 w, 128 + 32 w + 32) of every 256-column chunk
   f32x16 acc[kMaxChunks][2];
@@ -287,110 +313,180 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_de_kernel(BwdParams p) {
       for (int r = 0; r < 16; ++r) acc[ci][hb][r] = 0.0f;
 
   unsigned long long n_recomputed = 0, n_product = 0;
+  bool touched = false;
+  const bool use_list = IS_DE ? (p.shortcut != 0) : (p.filter_c != 0);
+  const int n_units = IS_DE ? p.nvc : p.ntg;          // what a pass scans: cells (dE) or row groups (dC)
+  const int seg_units = IS_DE ? kSegCells : kListCap;
 
-  for (int seg = 0; seg < p.nvc; seg += kListCap) {
-    const int seg_n = min(kListCap, p.nvc - seg);
-    // ---- which cells of this segment have to be recomputed ------------------------------------
-    if (p.shortcut) {
-      for (int j = tid; j < seg_n; j += kBwdThreads) {
-        const float cell = p.tile_max[static_cast<int64_t>(tg) * p.stat_cols + seg + j];
-        sFlag[j] = (cell - min_lse >= p.log_eps) ? 1 : 0;
-      }
-      __syncthreads();
-      if (tid < 32) {
-        const int t = meta.tgt[tid];
-        if (t >= 0) {
-          const int cell = t / 128 - seg;
-          if (cell >= 0 && cell < seg_n) sFlag[cell] = 1;
+  for (int seg = 0; seg < n_units; seg += seg_units) {
+    const int seg_n = min(seg_units, n_units - seg);
+    // ---- entries of this pass: class sub-blocks (dE) or row groups (dC), in increasing order --------
+    if (use_list) {
+      if (IS_DE) {
+        // a cell whose bound reaches eps needs all four sub-blocks; otherwise only those holding a target
+        for (int j = tid; j < seg_n; j += kBwdThreads) {
+          const float cell = p.tile_max[static_cast<int64_t>(own) * p.stat_cols + seg + j];
+          sFlag[j] = (cell - min_lse >= p.log_eps) ? 0xF : 0;
         }
+        __syncthreads();
+        if (tid < 32) {
+          const int t = meta.tgt[tid];
+          if (t >= 0) {
+            const int cell = t / 128 - seg;
+            if (cell >= 0 && cell < seg_n)
+              atomicOr(reinterpret_cast<unsigned int*>(sFlag) + (cell >> 2), (1u << ((t >> 5) & 3)) << ((cell & 3) * 8));
+          }
+        }
+        __syncthreads();
       }
-      __syncthreads();
       if (wave == 0) {  // ordered compaction: the accumulation order, hence the result, is fixed
         int n = 0;
         for (int base = 0; base < seg_n; base += 64) {
-          const bool f = (base + lane < seg_n) && (sFlag[base + lane] != 0);
-          const unsigned long long m = __ballot(f);
-          if (f) sList[n + __popcll(m & ((1ull << lane) - 1ull))] = seg + base + lane;
-          n += __popcll(m);
+          if (IS_DE) {
+            const int m = (base + lane < seg_n) ? sFlag[base + lane] : 0;
+            const int cnt = __popc(m);
+            int incl = cnt;  // inclusive prefix sum over the wave
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+              const int v = __shfl_up(incl, off, 64);
+              if (lane >= off) incl += v;
+            }
+            int pos = n + incl - cnt;
+#pragma unroll
+            for (int sb = 0; sb < 4; ++sb)
+              if ((m >> sb) & 1) sList[pos++] = (seg + base + lane) * 4 + sb;
+            n += __shfl(incl, 63, 64);
+          } else {
+            bool f = false;
+            if (base + lane < seg_n) {
+              const uint32_t w = p.kept_bits[static_cast<int64_t>(seg + base + lane) * p.bit_words + (own >> 5)];
+              f = ((w >> (own & 31)) & 1u) != 0u;
+            }
+            const unsigned long long m = __ballot(f);
+            if (f) sList[n + __popcll(m & ((1ull << lane) - 1ull))] = seg + base + lane;
+            n += __popcll(m);
+          }
         }
         if (lane == 0) sMisc[0] = n;
       }
       __syncthreads();
     }
-    const int list_n = p.shortcut ? sMisc[0] : seg_n;
+    const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
 
-    for (int li = 0; li < list_n; ++li) {
-      const int vc = p.shortcut ? sList[li] : seg + li;
-      // ---- class ids of the cell ---------------------------------------------------------------
-      if (tid < 128) {
-        const int64_t pos = static_cast<int64_t>(vc) * 128 + tid;
-        int cid = -1;
-        if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
-        sCid[tid] = cid;
+    for (int li = 0; li < list_n; li += 4) {
+      // ---- the virtual cell: up to four entries, 32 other-side rows each -------------------------------
+      if (IS_DE) {
+        if (tid < 128) {
+          const int k = li + (tid >> 5);
+          int cid = -1;
+          if (k < list_n) {
+            const int vg = use_list ? sList[k] : seg * 4 + k;
+            const int64_t pos = static_cast<int64_t>(vg) * 32 + (tid & 31);
+            if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
+          }
+          sCellCid[tid] = cid;
+        }
+      } else {
+        if (tid < 128) {
+          const int k = li + (tid >> 5);
+          int64_t i = p.b;  // no row
+          if (k < list_n) i = static_cast<int64_t>(use_list ? sList[k] : seg + k) * 32 + (tid & 31);
+          load_row_meta(p, i, tid, meta);
+        }
       }
       if (tid == 0) sMisc[1] = 0;
       __syncthreads();
+      const int* other_ids = IS_DE ? sCellCid : meta.row;
+      const int entry = li + wave;
+      const bool have_entry = entry < list_n;
+      const int entry_id = have_entry ? (use_list ? sList[entry] : (IS_DE ? seg * 4 + entry : seg + entry)) : -1;
 
-      // ---- logits^T (128 classes x 32 rows): wave w = classes [32 w, 32 w + 32) -----------------------
+      // ---- logits^T of (entry of this wave) x (own rows) over all of D --------------------------------------
       f32x16 s;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = 0.0f;
       {
-        StageLoader<128, ALIGNED> lc;
-        StageLoader<32, ALIGNED> le;
+        StageLoader<128, ALIGNED> lo;
+        StageLoader<32, ALIGNED> lw;
+        const uint16_t* other_base = IS_DE ? p.c : p.e;
+        const uint16_t* own_base = IS_DE ? p.e : p.c;
+        const int64_t other_sr = IS_DE ? p.stride_cv : p.stride_e;
+        const int64_t other_sc = IS_DE ? p.stride_cd : 1;
+        const int64_t own_sr = IS_DE ? p.stride_e : p.stride_cv;
+        const int64_t own_sc = IS_DE ? 1 : p.stride_cd;
         const int nstages = (D + kStageCols - 1) / kStageCols;
-        lc.load(sCid, p.c, p.stride_cv, p.stride_cd, 0, D, 0xfu);
-        le.load(meta.row, p.e, p.stride_e, 1, 0, D, 0x1u);
+        lo.load(other_ids, other_base, other_sr, other_sc, 0, D, 0xfu);
+        lw.load(own_ids, own_base, own_sr, own_sc, 0, D, 0x1u);
         for (int st = 0; st < nstages; ++st) {
-          lc.store(sC, 0xfu);
-          le.store(sE, 0x1u);
+          lo.store(sOther, 0xfu);
+          lw.store(sOwn, 0x1u);
           __syncthreads();
           if (st + 1 < nstages) {
-            lc.load(sCid, p.c, p.stride_cv, p.stride_cd, (st + 1) * kStageCols, D, 0xfu);
-            le.load(meta.row, p.e, p.stride_e, 1, (st + 1) * kStageCols, D, 0x1u);
+            lo.load(other_ids, other_base, other_sr, other_sc, (st + 1) * kStageCols, D, 0xfu);
+            lw.load(own_ids, own_base, own_sr, own_sc, (st + 1) * kStageCols, D, 0x1u);
           }
 #pragma unroll
           for (int kk = 0; kk < 16; ++kk) {
-            const auto a = stage_frag<T>(sC, wave * 32 + l32, kk * 2 + half);
-            const auto b = stage_frag<T>(sE, l32, kk * 2 + half);
-            s = Elem<T>::mfma(a, b, s);
+            // MFMA A operand = class rows, B operand = token rows
+            const auto fo = stage_frag<T>(sOther, wave * 32 + l32, kk * 2 + half);
+            const auto fw = stage_frag<T>(sOwn, l32, kk * 2 + half);
+            s = IS_DE ? Elem<T>::mfma(fo, fw, s) : Elem<T>::mfma(fw, fo, s);
           }
           __syncthreads();
         }
       }
 
-      // ---- dz, filter per 32 x 32 sub-tile ---------------------------------------------------------
+      // ---- dz of this wave's 32 x 32 block (lane = token row, registers = classes) ----------------------------
       {
-        const bool big = block_epilogue<T>(p, s, sCid + wave * 32, half, meta.lse2[l32], meta.g[l32], meta.h[l32],
-                                           meta.tgt[l32]);
-        const bool survives = (p.filter_eps < 0.0f) || (__ballot(big) != 0ull);
-        const bool live = (static_cast<int64_t>(vc) * 128 + wave * 32 < p.v);
-        const bool use = live && (survives || !p.filter_e);
+        const int mrow = IS_DE ? l32 : wave * 32 + l32;  // metadata slot of this lane's token row
+        const int* cid32 = IS_DE ? sCellCid + wave * 32 : sOwnCid;
+        const bool big = block_epilogue<T>(p, s, cid32, half, meta.lse2[mrow], meta.g[mrow], meta.h[mrow], meta.tgt[mrow]);
+        bool use = have_entry;
+        if (IS_DE) {
+          const bool survives = (p.filter_eps < 0.0f) || (__ballot(big) != 0ull);
+          const bool live = have_entry && (static_cast<int64_t>(entry_id) * 32 < p.v);
+          use = live && (survives || !p.filter_e);
+          if (lane == 0 && live && survives) atomicOr(&sBits[entry_id >> 5], 1u << (entry_id & 31));
+          if (lane == 0 && live) n_recomputed += 1;
+        }
         if (use) {
+          if (IS_DE) {
+            // dz [own row = lane][class of the cell]: four consecutive classes per store
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const int cls = wave * 32 + 8 * r4 + 4 * half;
-            uint2 pk;
-            pk.x = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 0])) |
-                   (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 1])) << 16);
-            pk.y = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 2])) |
-                   (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 3])) << 16);
-            *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((cls >> 3) ^ (l32 & 7)) << 4) | ((cls & 7) << 1))) = pk;
+            for (int r4 = 0; r4 < 4; ++r4) {
+              const int k = wave * 32 + 8 * r4 + 4 * half;
+              uint2 pk;
+              pk.x = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 0])) |
+                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 1])) << 16);
+              pk.y = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 2])) |
+                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 3])) << 16);
+              *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((k >> 3) ^ (l32 & 7)) << 4) | ((k & 7) << 1))) = pk;
+            }
+          } else {
+            // dz [own class][row of the cell = lane]; row sums feed dBias
+            const int k = wave * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
+              *reinterpret_cast<uint16_t*>(sDz + cls * 256 + ((((k >> 3) ^ (cls & 7)) << 4) | ((k & 7) << 1))) =
+                  Elem<T>::from_float(s[r]);
+              float colsum = s[r];
+#pragma unroll
+              for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
+              if (l32 == 0) sDb[wave * 32 + cls] += colsum;  // one writer per slot: deterministic
+            }
           }
           if (lane == 0) atomicOr(&sMisc[1], 1 << wave);
         }
-        if (lane == 0 && live && survives) {
-          const int vg = vc * 4 + wave;
-          atomicOr(&sBits[vg >> 5], 1u << (vg & 31));
-        }
-        if (lane == 0 && live) n_recomputed += 1;
       }
       __syncthreads();
       const uint32_t mask = static_cast<uint32_t>(sMisc[1]);
-      if (!write_de || mask == 0u) continue;
+      if (mask == 0u) continue;
+      touched = true;
       if (tid == 0) n_product += __popc(mask);
+      if (!write_out) continue;
 
-      // ---- dE^T (D x 32 rows) += C_cell^T . dz^T, 256 columns of D per stage ---------------------------
+      // ---- own_grad^T (D x 32) += Other_cell^T . dz, 256 columns of D per stage ------------------------------------
       typename Elem<T>::vec8 bz[8];
 #pragma unroll
       for (int kk = 0; kk < 8; ++kk) {
@@ -398,21 +494,23 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_de_kernel(BwdParams p) {
         bz[kk] = __builtin_bit_cast(typename Elem<T>::vec8, v);
       }
       {
-        StageLoader<128, ALIGNED> lc;
-        lc.load(sCid, p.c, p.stride_cv, p.stride_cd, d_begin, d_end, mask);
+        StageLoader<128, ALIGNED> lo;
+        const uint16_t* other_base = IS_DE ? p.c : p.e;
+        const int64_t other_sr = IS_DE ? p.stride_cv : p.stride_e;
+        const int64_t other_sc = IS_DE ? p.stride_cd : 1;
+        lo.load(other_ids, other_base, other_sr, other_sc, d_begin, d_end, mask);
 #pragma unroll
         for (int ci = 0; ci < kMaxChunks; ++ci) {
           if (ci < nchunks) {
-            lc.store(sC, mask);
+            lo.store(sOther, mask);
             __syncthreads();
-            if (ci + 1 < nchunks)
-              lc.load(sCid, p.c, p.stride_cv, p.stride_cd, d_begin + (ci + 1) * kStageCols, d_end, mask);
+            if (ci + 1 < nchunks) lo.load(other_ids, other_base, other_sr, other_sc, d_begin + (ci + 1) * kStageCols, d_end, mask);
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
               if ((mask >> (kk >> 1)) & 1u) {
 #pragma unroll
                 for (int hb = 0; hb < 2; ++hb) {
-                  const auto a = stage_frag_transposed<T>(sC, kk * 16 + half * 8, hb * 128 + wave * 32 + l32);
+                  const auto a = stage_frag_transposed<T>(sOther, kk * 16 + half * 8, hb * 128 + wave * 32 + l32);
                   acc[ci][hb] = Elem<T>::mfma(a, bz[kk], acc[ci][hb]);
                 }
               }
@@ -424,226 +522,43 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_de_kernel(BwdParams p) {
     }
   }
 
-  // ---- write the rows of this group, the bit row and the counters --------------------------------
-  if (write_de) {
-    const int row = meta.row[l32];
-    if (row >= 0) {
+  // ---- write the own rows once; rows nobody touched keep the caller's zeros ------------------------------
+  if (write_out && touched) {
+    const int id = own_ids[l32];
+    if (id >= 0) {
 #pragma unroll
       for (int ci = 0; ci < kMaxChunks; ++ci) {
         if (ci < nchunks) {
 #pragma unroll
-          for (int hb = 0; hb < 2; ++hb)
-            store_rows<T>(acc[ci][hb], p.d_e, p.de_fp32 != 0, p.vec_e != 0, static_cast<int64_t>(row) * p.stride_e, 1,
-                          d_begin + ci * kStageCols + hb * 128 + wave * 32, half, d_end);
+          for (int hb = 0; hb < 2; ++hb) {
+            const int col0 = d_begin + ci * kStageCols + hb * 128 + wave * 32;
+            if (IS_DE)
+              store_rows<T>(acc[ci][hb], p.d_e, p.de_fp32 != 0, p.vec_e != 0, static_cast<int64_t>(id) * p.stride_e, 1,
+                            col0, half, d_end);
+            else
+              store_rows<T>(acc[ci][hb], p.d_c, p.dc_fp32 != 0, p.vec_c != 0, static_cast<int64_t>(id) * p.stride_cv,
+                            p.stride_cd, col0, half, d_end);
+          }
         }
       }
     }
   }
   if (slice == 0) {
-    if (p.kept_bits != nullptr)
-      for (int w = tid; w < p.bit_words; w += kBwdThreads)
-        p.kept_bits[static_cast<int64_t>(tg) * p.bit_words + w] = sBits[w];
-    if (p.counters != nullptr) {
-      // every wave counted the sub-tiles it recomputed; thread 0 those that entered a product
-      if (lane == 0 && n_recomputed) atomicAdd(p.counters + 1, n_recomputed);
-      if (tid == 0 && n_product) atomicAdd(p.counters + 2, n_product);
-      if (tid == 0 && blockIdx.x == 0)
-        atomicAdd(p.counters + 0, static_cast<unsigned long long>(p.ntg) * static_cast<unsigned long long>(p.nvg));
+    if (IS_DE) {
+      if (p.kept_bits != nullptr)
+        for (int w = tid; w < p.bit_words; w += kBwdThreads)
+          p.kept_bits[static_cast<int64_t>(own) * p.bit_words + w] = sBits[w];
+      if (p.counters != nullptr) {
+        if (lane == 0 && n_recomputed) atomicAdd(p.counters + 1, n_recomputed);
+        if (tid == 0 && n_product) atomicAdd(p.counters + 2, n_product);
+        if (tid == 0 && blockIdx.x == 0)
+          atomicAdd(p.counters + 0, static_cast<unsigned long long>(p.ntg) * static_cast<unsigned long long>(p.nvg));
+      }
+    } else {
+      if (p.d_bias != nullptr && touched && tid < 32 && sOwnCid[tid] >= 0)
+        p.d_bias[sOwnCid[tid]] = (sDb[tid] + sDb[32 + tid]) + (sDb[64 + tid] + sDb[96 + tid]);
+      if (p.counters != nullptr && tid == 0 && n_product) atomicAdd(p.counters + 3, n_product);
     }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// dC / dBias: workgroup = (class group of 32, slice of D)
-// ---------------------------------------------------------------------------------------------
-constexpr int kDcOffC = 0;                   // 16 KB  C stage: 32 classes x 256 columns
-constexpr int kDcOffE = 16 * 1024;           // 16 KB  E stage: 32 rows x 256 columns
-constexpr int kDcOffPart = 32 * 1024;        // 16 KB  partial logits of the four K quarters
-constexpr int kDcOffDz = 48 * 1024;          //  2 KB  dz [class][row], 64 bytes per row
-constexpr int kDcOffList = 50 * 1024;        // 16 KB  row-group list
-constexpr int kDcOffMeta = 66 * 1024;
-constexpr int kDcLdsBytes = kDcOffMeta + 5 * 128 + 128 + 128 + 64;
-
-template <typename T, bool ALIGNED>
-__global__ __launch_bounds__(kBwdThreads, 1) void bwd_dc_kernel(BwdParams p) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sC = smem + kDcOffC;
-  unsigned char* sE = smem + kDcOffE;
-  float* sPart = reinterpret_cast<float*>(smem + kDcOffPart);
-  unsigned char* sDz = smem + kDcOffDz;
-  int* sList = reinterpret_cast<int*>(smem + kDcOffList);
-  RowMeta meta;
-  meta.row = reinterpret_cast<int*>(smem + kDcOffMeta);
-  meta.tgt = meta.row + 32;
-  meta.lse2 = reinterpret_cast<float*>(meta.tgt + 32);
-  meta.g = meta.lse2 + 32;
-  meta.h = meta.g + 32;
-  int* sCid = reinterpret_cast<int*>(meta.h + 32);     // [32]
-  float* sDb = reinterpret_cast<float*>(sCid + 32);    // [32] dBias of the group
-  int* sMisc = reinterpret_cast<int*>(sDb + 32);
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int l32 = lane & 31;
-  const int half = lane >> 5;
-  const int vg = blockIdx.x / p.nslices;
-  const int slice = blockIdx.x % p.nslices;
-  const int d_begin = slice * p.dslice;
-  const int d_end = min(static_cast<int>(p.d), d_begin + p.dslice);
-  const int nchunks = (d_end - d_begin + kStageCols - 1) / kStageCols;
-  const int D = static_cast<int>(p.d);
-  const bool write_dc = (p.d_c != nullptr);
-  const bool use_bits = (p.filter_c != 0);
-
-  if (tid < 32) {
-    const int64_t pos = static_cast<int64_t>(vg) * 32 + tid;
-    int cid = -1;
-    if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
-    sCid[tid] = cid;
-    sDb[tid] = 0.0f;
-  }
-  __syncthreads();
-
-  f32x16 acc[kMaxChunks][2];
-#pragma unroll
-  for (int ci = 0; ci < kMaxChunks; ++ci)
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ci][hb][r] = 0.0f;
-  unsigned long long n_product = 0;
-  bool touched = false;
-
-  for (int seg = 0; seg < p.ntg; seg += kListCap) {
-    const int seg_n = min(kListCap, p.ntg - seg);
-    if (use_bits) {
-      if (wave == 0) {
-        int n = 0;
-        for (int base = 0; base < seg_n; base += 64) {
-          bool f = false;
-          if (base + lane < seg_n) {
-            const uint32_t w = p.kept_bits[static_cast<int64_t>(seg + base + lane) * p.bit_words + (vg >> 5)];
-            f = ((w >> (vg & 31)) & 1u) != 0u;
-          }
-          const unsigned long long m = __ballot(f);
-          if (f) sList[n + __popcll(m & ((1ull << lane) - 1ull))] = seg + base + lane;
-          n += __popcll(m);
-        }
-        if (lane == 0) sMisc[0] = n;
-      }
-      __syncthreads();
-    }
-    const int list_n = use_bits ? sMisc[0] : seg_n;
-
-    for (int li = 0; li < list_n; ++li) {
-      const int tg = use_bits ? sList[li] : seg + li;
-      if (tid < 32) load_row_meta(p, static_cast<int64_t>(tg) * 32 + tid, tid, meta);
-      __syncthreads();
-
-      // ---- logits^T (32 classes x 32 rows): the 4 waves split every stage 4 ways along K ------------
-      f32x16 s;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-      {
-        StageLoader<32, ALIGNED> lc, le;
-        const int nstages = (D + kStageCols - 1) / kStageCols;
-        lc.load(sCid, p.c, p.stride_cv, p.stride_cd, 0, D, 0x1u);
-        le.load(meta.row, p.e, p.stride_e, 1, 0, D, 0x1u);
-        for (int st = 0; st < nstages; ++st) {
-          lc.store(sC, 0x1u);
-          le.store(sE, 0x1u);
-          __syncthreads();
-          if (st + 1 < nstages) {
-            lc.load(sCid, p.c, p.stride_cv, p.stride_cd, (st + 1) * kStageCols, D, 0x1u);
-            le.load(meta.row, p.e, p.stride_e, 1, (st + 1) * kStageCols, D, 0x1u);
-          }
-#pragma unroll
-          for (int k4 = 0; k4 < 4; ++k4) {
-            const int kk = wave * 4 + k4;
-            const auto a = stage_frag<T>(sC, l32, kk * 2 + half);
-            const auto b = stage_frag<T>(sE, l32, kk * 2 + half);
-            s = Elem<T>::mfma(a, b, s);
-          }
-          __syncthreads();
-        }
-      }
-      if (wave != 0) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sPart[(wave * 16 + r) * 64 + lane] = s[r];
-      }
-      __syncthreads();
-      if (wave == 0) {
-#pragma unroll
-        for (int w = 1; w < 4; ++w)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[r] += sPart[(w * 16 + r) * 64 + lane];
-        block_epilogue<T>(p, s, sCid, half, meta.lse2[l32], meta.g[l32], meta.h[l32], meta.tgt[l32]);
-        // dz [class][row] for the dC product; row sums for dBias
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
-          *reinterpret_cast<uint16_t*>(sDz + cls * 64 + l32 * 2) = Elem<T>::from_float(s[r]);
-          float colsum = s[r];
-#pragma unroll
-          for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
-          if (l32 == 0) sDb[cls] += colsum;
-        }
-      }
-      __syncthreads();
-      touched = true;
-      if (tid == 0) n_product += 1;
-      if (!write_dc) continue;
-
-      // ---- dC^T (D x 32 classes) += E_group^T . dz, 256 columns of D per stage -----------------------------
-      typename Elem<T>::vec8 bz[2];
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const uint4 v = *reinterpret_cast<const uint4*>(sDz + l32 * 64 + ((kk * 2 + half) << 4));
-        bz[kk] = __builtin_bit_cast(typename Elem<T>::vec8, v);
-      }
-      {
-        StageLoader<32, ALIGNED> le;
-        le.load(meta.row, p.e, p.stride_e, 1, d_begin, d_end, 0x1u);
-#pragma unroll
-        for (int ci = 0; ci < kMaxChunks; ++ci) {
-          if (ci < nchunks) {
-            le.store(sE, 0x1u);
-            __syncthreads();
-            if (ci + 1 < nchunks) le.load(meta.row, p.e, p.stride_e, 1, d_begin + (ci + 1) * kStageCols, d_end, 0x1u);
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-              for (int hb = 0; hb < 2; ++hb) {
-                const auto a = stage_frag_transposed<T>(sE, kk * 16 + half * 8, hb * 128 + wave * 32 + l32);
-                acc[ci][hb] = Elem<T>::mfma(a, bz[kk], acc[ci][hb]);
-              }
-            }
-            __syncthreads();
-          }
-        }
-      }
-    }
-  }
-
-  // Rows nobody touched keep the caller's zeros.
-  if (write_dc && touched) {
-    const int cid = sCid[l32];
-    if (cid >= 0) {
-#pragma unroll
-      for (int ci = 0; ci < kMaxChunks; ++ci) {
-        if (ci < nchunks) {
-#pragma unroll
-          for (int hb = 0; hb < 2; ++hb)
-            store_rows<T>(acc[ci][hb], p.d_c, p.dc_fp32 != 0, p.vec_c != 0, static_cast<int64_t>(cid) * p.stride_cv,
-                          p.stride_cd, d_begin + ci * kStageCols + hb * 128 + wave * 32, half, d_end);
-        }
-      }
-    }
-  }
-  if (slice == 0) {
-    if (p.d_bias != nullptr && touched && tid < 32 && sCid[tid] >= 0) p.d_bias[sCid[tid]] = sDb[tid];
-    if (p.counters != nullptr && tid == 0 && n_product) atomicAdd(p.counters + 3, n_product);
   }
 }
 
@@ -680,7 +595,7 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
   if (n_rows >= (int64_t(1) << 31) || v >= (int64_t(1) << 31) - 512 || d > (1 << 24)) return CCE_ERR_INVALID_ARGUMENT;
   if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
   if (d_e == nullptr && d_c == nullptr && d_bias == nullptr) return CCE_OK;
-  if (bit_words_for(v) > kDeMaxBitWords) return CCE_ERR_INVALID_ARGUMENT;
+  if (bit_words_for(v) > kMaxBitWords) return CCE_ERR_INVALID_ARGUMENT;
 
   BwdParams p;
   p.e = static_cast<const uint16_t*>(e);
@@ -761,11 +676,11 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
     if (d_e == nullptr) { q.nslices = 1; q.dslice = p.dslice; }
     p = q;
     if (dtype == CCE_DTYPE_BF16) {
-      if (aligned) CCE_LAUNCH((bwd_de_kernel<BF16, true>), kDeLdsBytes, grid);
-      else CCE_LAUNCH((bwd_de_kernel<BF16, false>), kDeLdsBytes, grid);
+      if (aligned) CCE_LAUNCH((bwd_owner_kernel<BF16, true, true>), kBwdLdsBytes, grid);
+      else CCE_LAUNCH((bwd_owner_kernel<BF16, false, true>), kBwdLdsBytes, grid);
     } else {
-      if (aligned) CCE_LAUNCH((bwd_de_kernel<F16, true>), kDeLdsBytes, grid);
-      else CCE_LAUNCH((bwd_de_kernel<F16, false>), kDeLdsBytes, grid);
+      if (aligned) CCE_LAUNCH((bwd_owner_kernel<F16, true, true>), kBwdLdsBytes, grid);
+      else CCE_LAUNCH((bwd_owner_kernel<F16, false, true>), kBwdLdsBytes, grid);
     }
     err = hipGetLastError();
     if (err != hipSuccess) return status_from_hip(err);
@@ -774,11 +689,11 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
     p.nslices = (d_c != nullptr) ? static_cast<int>((d + kMaxChunks * kStageCols - 1) / (kMaxChunks * kStageCols)) : 1;
     const unsigned grid = static_cast<unsigned>(p.nvg) * static_cast<unsigned>(p.nslices);
     if (dtype == CCE_DTYPE_BF16) {
-      if (aligned) CCE_LAUNCH((bwd_dc_kernel<BF16, true>), kDcLdsBytes, grid);
-      else CCE_LAUNCH((bwd_dc_kernel<BF16, false>), kDcLdsBytes, grid);
+      if (aligned) CCE_LAUNCH((bwd_owner_kernel<BF16, true, false>), kBwdLdsBytes, grid);
+      else CCE_LAUNCH((bwd_owner_kernel<BF16, false, false>), kBwdLdsBytes, grid);
     } else {
-      if (aligned) CCE_LAUNCH((bwd_dc_kernel<F16, true>), kDcLdsBytes, grid);
-      else CCE_LAUNCH((bwd_dc_kernel<F16, false>), kDcLdsBytes, grid);
+      if (aligned) CCE_LAUNCH((bwd_owner_kernel<F16, true, false>), kBwdLdsBytes, grid);
+      else CCE_LAUNCH((bwd_owner_kernel<F16, false, false>), kBwdLdsBytes, grid);
     }
   }
 #undef CCE_LAUNCH
