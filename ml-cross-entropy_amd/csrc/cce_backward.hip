@@ -562,6 +562,377 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fast variant of the ownership kernel (16-byte aligned rows, unit column stride, D % 128 == 0):
+// the same algorithm with direct global -> LDS loads (no staging registers, no LDS stores) and a
+// ring of three 128-column stages, so that two stages of HBM / L2 latency are always in flight.
+// Both phases of a trip are latency-bound, not MFMA-bound, which is why the depth of the load
+// pipeline is what matters here.
+//
+// Stage layout: 256-byte rows (128 columns), 16-byte chunks XOR-swizzled with (row & 15); one load
+// instruction of a wave fills 1 KB = 4 rows, lane l -> row (l >> 4), chunk slot (l & 15).  Other-side
+// block b = q * 4 + wave holds rows [4 b, 4 b + 4) of the 128-row virtual cell; own-side likewise for
+// its 32 rows.  A row id of -1 (no row) is fetched from row 0 of the matrix: the values are finite
+// and only ever meet a dz of exactly zero.
+// ---------------------------------------------------------------------------------------------
+constexpr int kFCols = 128;
+constexpr int kFRowBytes = 256;
+constexpr int kFOtherBytes = 128 * kFRowBytes;      // 32 KB
+constexpr int kFOwnBytes = 32 * kFRowBytes;         //  8 KB
+constexpr int kFStageBytes = kFOtherBytes + kFOwnBytes;
+constexpr int kFMaxChunks = 18;                     // 18 * 128 = 2304 columns of D per workgroup
+constexpr int kFOffDz = 3 * kFStageBytes;           // 120 KB
+constexpr int kFOffList = kFOffDz + 8 * 1024;       //   8 KB entry list (2048 entries)
+constexpr int kFOffFlag = kFOffList + 8 * 1024;     // 512 B
+constexpr int kFOffBits = kFOffFlag + 512;          //   8 KB
+constexpr int kFOffMeta = kFOffBits + kMaxBitWords * 4;
+constexpr int kFLdsBytes = kFOffMeta + 5 * kMetaRows * 4 + 32 * 4 + 128 * 4 + 128 * 4 + 64;
+constexpr int kFSegCells = 512;                     // dE: cells scanned per pass (<= 2048 entries)
+constexpr int kFListCap = 2048;
+static_assert(kFLdsBytes <= 160 * 1024, "LDS budget of gfx950");
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 fstage_frag(const unsigned char* lds, int row, int chunk) {
+  const uint4 v = *reinterpret_cast<const uint4*>(lds + row * kFRowBytes + ((chunk ^ (row & 15)) << 4));
+  return __builtin_bit_cast(typename Elem<T>::vec8, v);
+}
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const unsigned char* lds, int r0, int col) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const int ra = r0 + i, rb = r0 + i + 1;
+    const uint32_t lo = *reinterpret_cast<const uint16_t*>(
+        lds + ra * kFRowBytes + ((((col >> 3) ^ (ra & 15)) << 4) | ((col & 7) << 1)));
+    const uint32_t hi = *reinterpret_cast<const uint16_t*>(
+        lds + rb * kFRowBytes + ((((col >> 3) ^ (rb & 15)) << 4) | ((col & 7) << 1)));
+    w[i >> 1] = lo | (hi << 16);
+  }
+  return __builtin_bit_cast(typename Elem<T>::vec8, make_uint4(w[0], w[1], w[2], w[3]));
+}
+
+template <typename T, bool IS_DE>
+__global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* sDz = smem + kFOffDz;
+  int* sList = reinterpret_cast<int*>(smem + kFOffList);
+  unsigned char* sFlag = smem + kFOffFlag;
+  uint32_t* sBits = reinterpret_cast<uint32_t*>(smem + kFOffBits);
+  RowMeta meta;
+  meta.row = reinterpret_cast<int*>(smem + kFOffMeta);
+  meta.tgt = meta.row + kMetaRows;
+  meta.lse2 = reinterpret_cast<float*>(meta.tgt + kMetaRows);
+  meta.g = meta.lse2 + kMetaRows;
+  meta.h = meta.g + kMetaRows;
+  int* sOwnCid = reinterpret_cast<int*>(meta.h + kMetaRows);
+  int* sCellCid = sOwnCid + 32;
+  float* sDb = reinterpret_cast<float*>(sCellCid + 128);
+  int* sMisc = reinterpret_cast<int*>(sDb + 128);
+  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(smem));
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int own = blockIdx.x / p.nslices;
+  const int slice = blockIdx.x % p.nslices;
+  const int d_begin = slice * p.dslice;
+  const int d_end = min(static_cast<int>(p.d), d_begin + p.dslice);
+  const int nchunks = (d_end - d_begin) / kFCols;
+  const int D = static_cast<int>(p.d);
+  const int nstages = D / kFCols;
+  const bool write_out = IS_DE ? (p.d_e != nullptr) : (p.d_c != nullptr);
+
+  const uint16_t* other_base = IS_DE ? p.c : p.e;
+  const uint16_t* own_base = IS_DE ? p.e : p.c;
+  const int64_t other_sr = IS_DE ? p.stride_cv : p.stride_e;
+  const int64_t own_sr = IS_DE ? p.stride_e : p.stride_cv;
+  // element offset of the chunk this lane fetches inside a 128-column stage
+  const int lane_chunk = ((lane & 15) ^ ((4 * wave + (lane >> 4)) & 15)) * 8;
+
+  float my_lse = INFINITY;
+  if (IS_DE) {
+    if (tid < 32) my_lse = load_row_meta(p, static_cast<int64_t>(own) * 32 + tid, tid, meta);
+    if (wave == 0) {
+      const float mn = wave_min(my_lse);
+      if (lane == 0) reinterpret_cast<float*>(sMisc)[2] = mn;
+    }
+    for (int w = tid; w < p.bit_words; w += kBwdThreads) sBits[w] = 0u;
+  } else if (tid < 32) {
+    const int64_t pos = static_cast<int64_t>(own) * 32 + tid;
+    int cid = -1;
+    if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
+    sOwnCid[tid] = cid;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sDb[w * 32 + tid] = 0.0f;
+  }
+  __syncthreads();
+  const float min_lse = reinterpret_cast<float*>(sMisc)[2];
+  const int* own_ids = IS_DE ? meta.row : sOwnCid;
+
+  // own-side load pointers (2 per wave and stage), fixed for the whole kernel
+  const uint16_t* own_ptr[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int id = own_ids[4 * (q * 4 + wave) + (lane >> 4)];
+    own_ptr[q] = own_base + static_cast<int64_t>(id < 0 ? 0 : id) * own_sr + lane_chunk;
+  }
+
+  // wave w owns columns [32 w, 32 w + 32) of every 128-column chunk
+  f32x16 acc[kFMaxChunks];
+#pragma unroll
+  for (int ci = 0; ci < kFMaxChunks; ++ci)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[ci][r] = 0.0f;
+
+  unsigned long long n_recomputed = 0, n_product = 0;
+  bool touched = false;
+  const bool use_list = IS_DE ? (p.shortcut != 0) : (p.filter_c != 0);
+  const int n_units = IS_DE ? p.nvc : p.ntg;
+  const int seg_units = IS_DE ? kFSegCells : kFListCap;
+
+  for (int seg = 0; seg < n_units; seg += seg_units) {
+    const int seg_n = min(seg_units, n_units - seg);
+    if (use_list) {
+      if (IS_DE) {
+        for (int j = tid; j < seg_n; j += kBwdThreads) {
+          const float cell = p.tile_max[static_cast<int64_t>(own) * p.stat_cols + seg + j];
+          sFlag[j] = (cell - min_lse >= p.log_eps) ? 0xF : 0;
+        }
+        __syncthreads();
+        if (tid < 32) {
+          const int t = meta.tgt[tid];
+          if (t >= 0) {
+            const int cell = t / 128 - seg;
+            if (cell >= 0 && cell < seg_n)
+              atomicOr(reinterpret_cast<unsigned int*>(sFlag) + (cell >> 2), (1u << ((t >> 5) & 3)) << ((cell & 3) * 8));
+          }
+        }
+        __syncthreads();
+      }
+      if (wave == 0) {
+        int n = 0;
+        for (int base = 0; base < seg_n; base += 64) {
+          if (IS_DE) {
+            const int m = (base + lane < seg_n) ? sFlag[base + lane] : 0;
+            const int cnt = __popc(m);
+            int incl = cnt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+              const int v = __shfl_up(incl, off, 64);
+              if (lane >= off) incl += v;
+            }
+            int pos = n + incl - cnt;
+#pragma unroll
+            for (int sb = 0; sb < 4; ++sb)
+              if ((m >> sb) & 1) sList[pos++] = (seg + base + lane) * 4 + sb;
+            n += __shfl(incl, 63, 64);
+          } else {
+            bool f = false;
+            if (base + lane < seg_n) {
+              const uint32_t w = p.kept_bits[static_cast<int64_t>(seg + base + lane) * p.bit_words + (own >> 5)];
+              f = ((w >> (own & 31)) & 1u) != 0u;
+            }
+            const unsigned long long m = __ballot(f);
+            if (f) sList[n + __popcll(m & ((1ull << lane) - 1ull))] = seg + base + lane;
+            n += __popcll(m);
+          }
+        }
+        if (lane == 0) sMisc[0] = n;
+      }
+      __syncthreads();
+    }
+    const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
+
+    for (int li = 0; li < list_n; li += 4) {
+      if (IS_DE) {
+        if (tid < 128) {
+          const int k = li + (tid >> 5);
+          int cid = -1;
+          if (k < list_n) {
+            const int vg = use_list ? sList[k] : seg * 4 + k;
+            const int64_t pos = static_cast<int64_t>(vg) * 32 + (tid & 31);
+            if (pos < p.v) cid = p.vocab_order ? p.vocab_order[pos] : static_cast<int>(pos);
+          }
+          sCellCid[tid] = cid;
+        }
+      } else {
+        if (tid < 128) {
+          const int k = li + (tid >> 5);
+          int64_t i = p.b;
+          if (k < list_n) i = static_cast<int64_t>(use_list ? sList[k] : seg + k) * 32 + (tid & 31);
+          load_row_meta(p, i, tid, meta);
+        }
+      }
+      if (tid == 0) sMisc[1] = 0;
+      __syncthreads();
+      const int* other_ids = IS_DE ? sCellCid : meta.row;
+      const int entry = li + wave;
+      const bool have_entry = entry < list_n;
+      const int entry_id = have_entry ? (use_list ? sList[entry] : (IS_DE ? seg * 4 + entry : seg + entry)) : -1;
+
+      // other-side load pointers of this trip (8 per wave and stage)
+      const uint16_t* other_ptr[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int id = other_ids[4 * (q * 4 + wave) + (lane >> 4)];
+        other_ptr[q] = other_base + static_cast<int64_t>(id < 0 ? 0 : id) * other_sr + lane_chunk;
+      }
+      auto issue_stage = [&](int col0, int slot, bool with_own) {
+        const unsigned base = lds_base + slot * kFStageBytes;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
+        if (with_own) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + kFOtherBytes + (q * 4 + wave) * 1024);
+        }
+      };
+
+      // ---- logits^T of (entry of this wave) x (own rows): 10 loads per wave and stage, two stages ahead ----
+      f32x16 s;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+      const int last_col = (nstages - 1) * kFCols;
+      issue_stage(0, 0, true);
+      issue_stage(min(kFCols, last_col), 1, true);
+#pragma unroll 1
+      for (int st = 0; st < nstages; ++st) {
+        asm volatile("s_waitcnt vmcnt(10)" ::: "memory");  // all but the newest stage have landed
+        __syncthreads();                                   // ... for every wave; stage st - 1 is consumed
+        issue_stage(min((st + 2) * kFCols, last_col), (st + 2) % 3, true);
+        const unsigned char* so = smem + (st % 3) * kFStageBytes;
+        const unsigned char* sw = so + kFOtherBytes;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const auto fo = fstage_frag<T>(so, wave * 32 + l32, kk * 2 + half);
+          const auto fw = fstage_frag<T>(sw, l32, kk * 2 + half);
+          s = IS_DE ? Elem<T>::mfma(fo, fw, s) : Elem<T>::mfma(fw, fo, s);
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the two unused prefetches
+      __syncthreads();
+      // first two stages of the product phase, in flight during the epilogue
+      const int last_chunk_col = d_begin + (nchunks - 1) * kFCols;
+      issue_stage(d_begin, 0, false);
+      issue_stage(min(d_begin + kFCols, last_chunk_col), 1, false);
+
+      // ---- dz of this wave's 32 x 32 block (lane = token row, registers = classes) ----------------------------
+      {
+        const int mrow = IS_DE ? l32 : wave * 32 + l32;
+        const int* cid32 = IS_DE ? sCellCid + wave * 32 : sOwnCid;
+        const bool big = block_epilogue<T>(p, s, cid32, half, meta.lse2[mrow], meta.g[mrow], meta.h[mrow], meta.tgt[mrow]);
+        bool use = have_entry;
+        if (IS_DE) {
+          const bool survives = (p.filter_eps < 0.0f) || (__ballot(big) != 0ull);
+          const bool live = have_entry && (static_cast<int64_t>(entry_id) * 32 < p.v);
+          use = live && (survives || !p.filter_e);
+          if (lane == 0 && live && survives) atomicOr(&sBits[entry_id >> 5], 1u << (entry_id & 31));
+          if (lane == 0 && live) n_recomputed += 1;
+        }
+        if (use) {
+          if (IS_DE) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+              const int k = wave * 32 + 8 * r4 + 4 * half;
+              uint2 pk;
+              pk.x = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 0])) |
+                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 1])) << 16);
+              pk.y = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 2])) |
+                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 3])) << 16);
+              *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((k >> 3) ^ (l32 & 7)) << 4) | ((k & 7) << 1))) = pk;
+            }
+          } else {
+            const int k = wave * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
+              *reinterpret_cast<uint16_t*>(sDz + cls * 256 + ((((k >> 3) ^ (cls & 7)) << 4) | ((k & 7) << 1))) =
+                  Elem<T>::from_float(s[r]);
+              float colsum = s[r];
+#pragma unroll
+              for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
+              if (l32 == 0) sDb[wave * 32 + cls] += colsum;
+            }
+          }
+          if (lane == 0) atomicOr(&sMisc[1], 1 << wave);
+        }
+      }
+      __syncthreads();
+      const uint32_t mask = static_cast<uint32_t>(sMisc[1]);
+      const bool product = write_out && (mask != 0u);
+      if (mask != 0u) {
+        touched = true;
+        if (tid == 0) n_product += __popc(mask);
+      }
+
+      // ---- own_grad^T (D x 32) += Other_cell^T . dz, 128 columns of D per stage --------------------------------------
+      typename Elem<T>::vec8 bz[8];
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const uint4 v = *reinterpret_cast<const uint4*>(sDz + l32 * 256 + (((kk * 2 + half) ^ (l32 & 7)) << 4));
+        bz[kk] = __builtin_bit_cast(typename Elem<T>::vec8, v);
+      }
+      if (product) {
+#pragma unroll
+        for (int ci = 0; ci < kFMaxChunks; ++ci) {
+          if (ci < nchunks) {
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            __syncthreads();
+            issue_stage(min(d_begin + (ci + 2) * kFCols, last_chunk_col), (ci + 2) % 3, false);
+            const unsigned char* so = smem + (ci % 3) * kFStageBytes;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+              if ((mask >> (kk >> 1)) & 1u) {
+                const auto a = fstage_frag_transposed<T>(so, kk * 16 + half * 8, wave * 32 + l32);
+                acc[ci] = Elem<T>::mfma(a, bz[kk], acc[ci]);
+              }
+            }
+          }
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain before the ring is refilled
+      __syncthreads();
+    }
+  }
+
+  if (write_out && touched) {
+    const int id = own_ids[l32];
+    if (id >= 0) {
+#pragma unroll
+      for (int ci = 0; ci < kFMaxChunks; ++ci) {
+        if (ci < nchunks) {
+          const int col0 = d_begin + ci * kFCols + wave * 32;
+          if (IS_DE)
+            store_rows<T>(acc[ci], p.d_e, p.de_fp32 != 0, p.vec_e != 0, static_cast<int64_t>(id) * p.stride_e, 1, col0,
+                          half, d_end);
+          else
+            store_rows<T>(acc[ci], p.d_c, p.dc_fp32 != 0, p.vec_c != 0, static_cast<int64_t>(id) * p.stride_cv,
+                          p.stride_cd, col0, half, d_end);
+        }
+      }
+    }
+  }
+  if (slice == 0) {
+    if (IS_DE) {
+      if (p.kept_bits != nullptr)
+        for (int w = tid; w < p.bit_words; w += kBwdThreads)
+          p.kept_bits[static_cast<int64_t>(own) * p.bit_words + w] = sBits[w];
+      if (p.counters != nullptr) {
+        if (lane == 0 && n_recomputed) atomicAdd(p.counters + 1, n_recomputed);
+        if (tid == 0 && n_product) atomicAdd(p.counters + 2, n_product);
+        if (tid == 0 && blockIdx.x == 0)
+          atomicAdd(p.counters + 0, static_cast<unsigned long long>(p.ntg) * static_cast<unsigned long long>(p.nvg));
+      }
+    } else {
+      if (p.d_bias != nullptr && touched && tid < 32 && sOwnCid[tid] >= 0)
+        p.d_bias[sOwnCid[tid]] = (sDb[tid] + sDb[32 + tid]) + (sDb[64 + tid] + sDb[96 + tid]);
+      if (p.counters != nullptr && tid == 0 && n_product) atomicAdd(p.counters + 3, n_product);
+    }
+  }
+}
+
 }  // namespace cce
 
 using namespace cce;
@@ -661,6 +1032,8 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
 
   const bool aligned = aligned16(e) && aligned16(c) && (d % 8 == 0) && (stride_e % 8 == 0) &&
                        (stride_cv % 8 == 0) && (stride_cd == 1);
+  // The fast kernels want whole 128-column stages, also inside every slice of D.
+  const bool fast = aligned && (d % kFCols == 0);
   hipError_t err;
 #define CCE_LAUNCH(KERN, LDS, GRID)                                                                 \
   do {                                                                                              \
@@ -668,34 +1041,34 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                  \
                               hipFuncAttributeMaxDynamicSharedMemorySize, LDS);                     \
     if (err != hipSuccess) return status_from_hip(err);                                             \
-    hipLaunchKernelGGL(kern, dim3(GRID), dim3(kBwdThreads), LDS, stream, p);                                \
+    hipLaunchKernelGGL(kern, dim3(GRID), dim3(kBwdThreads), LDS, stream, p);                        \
   } while (0)
+#define CCE_LAUNCH_OWNER(IS_DE_, GRID)                                                              \
+  do {                                                                                              \
+    if (dtype == CCE_DTYPE_BF16) {                                                                  \
+      if (fast) CCE_LAUNCH((bwd_owner_fast_kernel<BF16, IS_DE_>), kFLdsBytes, GRID);                \
+      else if (aligned) CCE_LAUNCH((bwd_owner_kernel<BF16, true, IS_DE_>), kBwdLdsBytes, GRID);     \
+      else CCE_LAUNCH((bwd_owner_kernel<BF16, false, IS_DE_>), kBwdLdsBytes, GRID);                 \
+    } else {                                                                                        \
+      if (fast) CCE_LAUNCH((bwd_owner_fast_kernel<F16, IS_DE_>), kFLdsBytes, GRID);                 \
+      else if (aligned) CCE_LAUNCH((bwd_owner_kernel<F16, true, IS_DE_>), kBwdLdsBytes, GRID);      \
+      else CCE_LAUNCH((bwd_owner_kernel<F16, false, IS_DE_>), kBwdLdsBytes, GRID);                  \
+    }                                                                                               \
+  } while (0)
+  const int full_slices = p.nslices;
   if (need_de_pass) {
-    const unsigned grid = static_cast<unsigned>(p.ntg) * static_cast<unsigned>(d_e != nullptr ? p.nslices : 1);
-    BwdParams q = p;
-    if (d_e == nullptr) { q.nslices = 1; q.dslice = p.dslice; }
-    p = q;
-    if (dtype == CCE_DTYPE_BF16) {
-      if (aligned) CCE_LAUNCH((bwd_owner_kernel<BF16, true, true>), kBwdLdsBytes, grid);
-      else CCE_LAUNCH((bwd_owner_kernel<BF16, false, true>), kBwdLdsBytes, grid);
-    } else {
-      if (aligned) CCE_LAUNCH((bwd_owner_kernel<F16, true, true>), kBwdLdsBytes, grid);
-      else CCE_LAUNCH((bwd_owner_kernel<F16, false, true>), kBwdLdsBytes, grid);
-    }
+    p.nslices = (d_e != nullptr) ? full_slices : 1;
+    const unsigned grid = static_cast<unsigned>(p.ntg) * static_cast<unsigned>(p.nslices);
+    CCE_LAUNCH_OWNER(true, grid);
     err = hipGetLastError();
     if (err != hipSuccess) return status_from_hip(err);
   }
   if (need_dc_pass) {
-    p.nslices = (d_c != nullptr) ? static_cast<int>((d + kMaxChunks * kStageCols - 1) / (kMaxChunks * kStageCols)) : 1;
+    p.nslices = (d_c != nullptr) ? full_slices : 1;
     const unsigned grid = static_cast<unsigned>(p.nvg) * static_cast<unsigned>(p.nslices);
-    if (dtype == CCE_DTYPE_BF16) {
-      if (aligned) CCE_LAUNCH((bwd_owner_kernel<BF16, true, false>), kBwdLdsBytes, grid);
-      else CCE_LAUNCH((bwd_owner_kernel<BF16, false, false>), kBwdLdsBytes, grid);
-    } else {
-      if (aligned) CCE_LAUNCH((bwd_owner_kernel<F16, true, false>), kBwdLdsBytes, grid);
-      else CCE_LAUNCH((bwd_owner_kernel<F16, false, false>), kBwdLdsBytes, grid);
-    }
+    CCE_LAUNCH_OWNER(false, grid);
   }
+#undef CCE_LAUNCH_OWNER
 #undef CCE_LAUNCH
   return status_from_hip(hipGetLastError());
 }
