@@ -22,6 +22,10 @@ for _p in (ROOT, os.path.join(ROOT, "ml-cross-entropy_amd")):
         sys.path.insert(0, _p)
 
 PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk x 2.4 GHz, dense
+# HBM bytes per launch of lse_forward_kernel at workload c2, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0
+# + WRITE_SIZE x 1.0, factors from a 1 GiB copy in the same runs; summary in profiles/).  A counter cannot be
+# read from inside this script, so the figure of the last profiled build is reported unless --traffic is given.
+MEASURED_TRAFFIC_BYTES = {"c2": 1.4185e10}
 
 
 def make_workload(name, device):
@@ -92,6 +96,10 @@ def main():
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one plain 1 GiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--traffic", type=float, default=None,
+                    help="HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc (reported as given)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives); use --gpus 1", file=sys.stderr)
@@ -119,6 +127,13 @@ def main():
         loss = linear_cross_entropy(e, c, t, softcap=w["softcap"], reduction="mean", impl="cce")
         loss.backward()
         return loss
+
+    if args.traffic_probe:
+        src = torch.empty((1 << 29,), dtype=torch.bfloat16, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -213,7 +228,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": fwd_tflops / PEAK_BF16_TFLOPS,
             "ms_per_launch": fwd_ms,
-            "traffic": None,
+            "traffic": args.traffic if args.traffic is not None else MEASURED_TRAFFIC_BYTES.get(w["name"]),
         },
     }
     if not args.no_cpu_baseline:

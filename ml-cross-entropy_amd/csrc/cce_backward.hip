@@ -612,6 +612,18 @@ __device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const u
   return __builtin_bit_cast(typename Elem<T>::vec8, make_uint4(w[0], w[1], w[2], w[3]));
 }
 
+// s_waitcnt vmcnt(n) for a wave-uniform n in {0, 2, 4, 6, 8, 10} (the immediate must be a constant).
+__device__ __forceinline__ void wait_vmcnt_upto(int n) {
+  switch (n) {
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+
 template <typename T, bool IS_DE>
 __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -780,10 +792,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         const int id = other_ids[4 * (q * 4 + wave) + (lane >> 4)];
         other_ptr[q] = other_base + static_cast<int64_t>(id < 0 ? 0 : id) * other_sr + lane_chunk;
       }
+      // Entries are packed at the front of a trip; the rows of absent ones are not fetched (loads
+      // 2 e and 2 e + 1 of a wave belong to entry e), so a short trip moves proportionally less data.
+      const int nent = min(4, list_n - li);
       auto issue_stage = [&](int col0, int slot, bool with_own) {
         const unsigned base = lds_base + slot * kFStageBytes;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
+        for (int q = 0; q < 8; ++q)
+          if ((q >> 1) < nent) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
         if (with_own) {
 #pragma unroll
           for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + kFOtherBytes + (q * 4 + wave) * 1024);
@@ -799,7 +815,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       issue_stage(min(kFCols, last_col), 1, true);
 #pragma unroll 1
       for (int st = 0; st < nstages; ++st) {
-        asm volatile("s_waitcnt vmcnt(10)" ::: "memory");  // all but the newest stage have landed
+        wait_vmcnt_upto(2 * nent + 2);  // all but the newest stage have landed
         __syncthreads();                                   // ... for every wave; stage st - 1 is consumed
         issue_stage(min((st + 2) * kFCols, last_col), (st + 2) % 3, true);
         const unsigned char* so = smem + (st % 3) * kFStageBytes;
@@ -878,7 +894,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 #pragma unroll
         for (int ci = 0; ci < kFMaxChunks; ++ci) {
           if (ci < nchunks) {
-            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            wait_vmcnt_upto(2 * nent);
             __syncthreads();
             issue_stage(min(d_begin + (ci + 2) * kFCols, last_chunk_col), (ci + 2) % 3, false);
             const unsigned char* so = smem + (ci % 3) * kFStageBytes;
