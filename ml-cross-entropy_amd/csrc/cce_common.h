@@ -462,9 +462,9 @@ struct FastLogitTile {
 // The loads are inline assembly (the compiler would otherwise wait for every outstanding load
 // before the next LDS read) and completion is tracked by hand: two LDS stages, one barrier per stage
 // placed before the last of the four 16-column steps.  At that barrier every wave has read its last
-// fragments of stage s, so the loads of stage s + 2 are issued into that LDS stage right there (a
-// full stage of MFMAs before they are awaited), and the first fragments of stage s + 1 are read
-// under the MFMAs of the last step.
+// fragments of stage s, so the loads of stage s + 2 may go into that LDS stage from there on; they are
+// spread over the next three steps, and the first fragments of stage s + 1 are read under the MFMAs
+// of the last step.
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ void lds_dma16(const void* gptr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr)
@@ -486,6 +486,10 @@ struct DmaLogitTile {
   static constexpr int NQE = TILE_T / 8 / NW;  // ... token rows
   static constexpr int NQ = NQC + NQE;
   static constexpr int NSTEP = kDmaBK / 16;
+  // The loads of a stage are issued in three groups, under the MFMAs of three consecutive steps:
+  // [0, QA) under step 3 of the stage before last, [QA, QB) and [QB, NQ) under steps 0 and 1 of the last.
+  static constexpr int QA = (NQ + 2) / 3;
+  static constexpr int QB = (2 * QA < NQ) ? 2 * QA : NQ;
   static_assert(TILE_V % (8 * NW) == 0 && TILE_T % (8 * NW) == 0, "blocks must divide over the waves");
   static_assert(NW % 2 == 0, "the swizzle of a lane must not depend on q");
   using vec8 = typename Elem<T>::vec8;
@@ -528,17 +532,50 @@ struct DmaLogitTile {
       for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
   }
 
-  // Issue the NQ loads of one stage (columns [k0, k0 + 64)) into LDS stage `stage_off`.
-  static __device__ __forceinline__ void issue(const uint16_t* const (&ptr)[NQ], int k0, unsigned lds_base,
-                                               int stage_off, int wave) {
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      const int blk = (q < NQC) ? (q * NW + wave) : (TILE_V / 8 + (q - NQC) * NW + wave);
-      lds_dma16(ptr[q] + k0, lds_base + stage_off + blk * 1024);
-    }
+  // Issue load q of one stage (columns [k0, k0 + 64)) into LDS stage `stage_off`.
+  static __device__ __forceinline__ void issue_one(const uint16_t* const (&ptr)[NQ], int q, int k0, unsigned lds_base,
+                                                   int stage_off, int wave) {
+    const int blk = (q < NQC) ? (q * NW + wave) : (TILE_V / 8 + (q - NQC) * NW + wave);
+    lds_dma16(ptr[q] + k0, lds_base + stage_off + blk * 1024);
   }
 
-  // D must be a multiple of 64.
+  // The MFMAs of one step with loads [Q0, Q1) of a stage issued between them, one after every second
+  // MFMA.  Measured: a burst of all NQ loads right after the barrier backs up the address path, the
+  // waves that issue last fall a third of a stage behind and everybody waits for them at the next
+  // barrier; a steady trickle keeps the waves together.
+  template <int Q0, int Q1>
+  static __device__ __forceinline__ void mma_loads(f32x16 (&acc)[WV][WT], const Frags& f,
+                                                   const uint16_t* const (&ptr)[NQ], int k0, unsigned lds_base,
+                                                   int stage_off, int wave) {
+    static_assert(Q1 - Q0 <= (WV * WT) / 2, "one load per two MFMAs");
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti) {
+        acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
+        const int idx = vi * WT + ti;
+        if ((idx & 1) && Q0 + idx / 2 < Q1) {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_one(ptr, Q0 + idx / 2, k0, lds_base, stage_off, wave);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+  }
+
+  // Start fetching a tile into the (idle) LDS ring: all of stage 0 and the first group of stage 1.
+  // Called before the epilogue of the previous tile, so that the next main loop starts with data in LDS.
+  static __device__ __forceinline__ void prefetch(const uint16_t* const (&ptr)[NQ], unsigned char* lds, int D) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+    const int last = (D / kDmaBK - 1) * kDmaBK;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) issue_one(ptr, q, 0, lds_base, 0, wave);
+#pragma unroll
+    for (int q = 0; q < QA; ++q) issue_one(ptr, q, min(kDmaBK, last), lds_base, STAGE_BYTES, wave);
+  }
+
+  // D must be a multiple of 64.  prefetch() with the same pointers must have been called, and nothing
+  // may have touched the LDS ring since.
   static __device__ __forceinline__ void run(f32x16 (&acc)[WV][WT], const uint16_t* const (&ptr)[NQ],
                                              unsigned char* lds, int D) {
     const int lane = threadIdx.x & 63;
@@ -561,10 +598,8 @@ struct DmaLogitTile {
 
     const int nk = D / kDmaBK;
     const int last = (nk - 1) * kDmaBK;
-    issue(ptr, 0, lds_base, 0, wave);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(QA) : "memory");  // stage 0 landed, stage 1 may be in flight
     __syncthreads();
-    issue(ptr, min(kDmaBK, last), lds_base, STAGE_BYTES, wave);
     Frags fa = read_frags(lds, 0, 0, coff0, eoff0, sw, half);
     Frags fb;
 
@@ -574,28 +609,29 @@ struct DmaLogitTile {
     for (int s = 0; s < nk; ++s) {
       const int cur = (s & 1) * STAGE_BYTES;
       const int nxt = STAGE_BYTES - cur;
+      const int k1 = min((s + 1) * kDmaBK, last);
+      const int k2 = min((s + 2) * kDmaBK, last);
       fb = read_frags(lds, cur, 1, coff0, eoff0, sw, half);
       __builtin_amdgcn_sched_barrier(0);
-      mma(acc, fa);  // step 0
+      mma_loads<QA, QB>(acc, fa, ptr, k1, lds_base, nxt, wave);  // step 0
       __builtin_amdgcn_sched_barrier(0);
       fa = read_frags(lds, cur, 2, coff0, eoff0, sw, half);
       __builtin_amdgcn_sched_barrier(0);
-      mma(acc, fb);  // step 1
+      mma_loads<QB, NQ>(acc, fb, ptr, k1, lds_base, nxt, wave);  // step 1
       __builtin_amdgcn_sched_barrier(0);
       fb = read_frags(lds, cur, 3, coff0, eoff0, sw, half);
       __builtin_amdgcn_sched_barrier(0);
       mma(acc, fa);  // step 2
       __builtin_amdgcn_sched_barrier(0);
-      // Stage s + 1 (issued a full stage ago) has landed for this wave; after the barrier, for every
-      // wave, and every wave holds its last fragments of stage s in registers: that LDS stage is free
-      // and the loads of stage s + 2 go into it.  A prefetch past the end re-reads the last stage
-      // (never consumed), which keeps the loop free of branches.
+      // Stage s + 1 (last loads issued two steps ago) has landed for this wave; after the barrier, for
+      // every wave, and every wave holds its last fragments of stage s in registers: that LDS stage is
+      // free and the first loads of stage s + 2 go into it.  A prefetch past the end re-reads the last
+      // stage (never consumed), which keeps the loop free of branches.
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      issue(ptr, min((s + 2) * kDmaBK, last), lds_base, cur, wave);
       fa = read_frags(lds, nxt, 0, coff0, eoff0, sw, half);
       __builtin_amdgcn_sched_barrier(0);
-      mma(acc, fb);  // step 3
+      mma_loads<0, QA>(acc, fb, ptr, k2, lds_base, cur, wave);  // step 3
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch

@@ -45,28 +45,44 @@ constexpr int kFwdBiasBytes = 2 * 256 * 4;  // two tiles' worth of per-class add
 // GENERAL adds a per-class addend staged in LDS: the bias (or 0), or -inf for a class past the end of
 // the vocabulary, which is masked AFTER soft-capping (soft-capping -inf would give -softcap, not -inf).
 // The plain variant is straight-line code with no loads.
-template <bool GENERAL>
-__device__ __forceinline__ float column_block_logits(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
-                                                     const float* addend, int half, float (&s2)[kFwdWV][16]) {
+template <bool GENERAL, bool CAP>
+__device__ __forceinline__ float column_block_logits_impl(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
+                                                          const float* addend, int half, float (&s2)[kFwdWV][16]) {
   float tm = -INFINITY;
 #pragma unroll
   for (int vi = 0; vi < kFwdWV; ++vi) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       float x = acc[vi][ti][r];
-      float th;
+      bool dead = false;
       if (GENERAL) {
         const float add = addend[vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
-        const bool dead = (add == -INFINITY);
-        const float y = softcap_log2(sc, dead ? 0.0f : x + add, th);
-        s2[vi][r] = dead ? -INFINITY : y;
-      } else {
-        s2[vi][r] = softcap_log2(sc, x, th);
+        dead = (add == -INFINITY);
+        x = dead ? 0.0f : x + add;
       }
+      float y;
+      if (CAP) {
+        // cap * log2(e) * tanh(x / cap), tanh(u) = 1 - 2 / (1 + exp(2 u))
+        const float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
+        const float w = __builtin_amdgcn_rcpf(1.0f + t);
+        y = fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
+      } else {
+        y = x * kLog2e;
+      }
+      s2[vi][r] = dead ? -INFINITY : y;
       tm = fmaxf(tm, s2[vi][r]);
     }
   }
   return tm;
+}
+
+// One uniform branch per column block: each arm is straight-line code over all 64 values, so the
+// independent exp2 / rcp chains of different values overlap.
+template <bool GENERAL>
+__device__ __forceinline__ float column_block_logits(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
+                                                     const float* addend, int half, float (&s2)[kFwdWV][16]) {
+  if (sc.on) return column_block_logits_impl<GENERAL, true>(sc, acc, ti, addend, half, s2);
+  return column_block_logits_impl<GENERAL, false>(sc, acc, ti, addend, half, s2);
 }
 
 // Kernel variants:
@@ -133,6 +149,15 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
     sum[ti] = 0.0f;
   }
 
+  auto set_class_pointers = [&](int64_t v0) {
+#pragma unroll
+    for (int q = 0; q < Fast::NQC; ++q) {
+      int64_t vr = v0 + Fast::row_of(q, wave, lane);
+      vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked in the epilogue
+      fptr[q] = p.c + vr * p.stride_cv + Fast::chunk_elems(wave, lane);
+    }
+  };
+
   for (int vt = vt_begin; vt < vt_end; ++vt) {
     const int64_t v0 = static_cast<int64_t>(vt) * Tile::TILE_V;
     float* addend = s_addend + (vt & 1) * kFwdTile;
@@ -148,13 +173,16 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
     }
     f32x16 acc[kFwdWV][kFwdWT];
     if (FAST) {
-#pragma unroll
-      for (int q = 0; q < Fast::NQC; ++q) {
-        int64_t vr = v0 + Fast::row_of(q, wave, lane);
-        vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked below
-        fptr[q] = p.c + vr * p.stride_cv + Fast::chunk_elems(wave, lane);
+      if (vt == vt_begin) {
+        set_class_pointers(v0);
+        Fast::prefetch(fptr, smem, static_cast<int>(p.d));
       }
       Fast::run(acc, fptr, smem, static_cast<int>(p.d));
+      if (vt + 1 < vt_end) {
+        // the ring is idle during the epilogue: start on the next tile now
+        set_class_pointers(v0 + Tile::TILE_V);
+        Fast::prefetch(fptr, smem, static_cast<int>(p.d));
+      }
     } else {
 #pragma unroll
       for (int q = 0; q < Tile::CLoader::NQ; ++q) {
