@@ -597,29 +597,38 @@ __device__ __forceinline__ typename Elem<T>::vec8 fstage_frag(const unsigned cha
   return __builtin_bit_cast(typename Elem<T>::vec8, v);
 }
 
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// MFMA operand whose reduction index runs over the stage rows k0 + 8 (lane >> 5) .. + 7, for column
+// col0 + (lane & 31): two LDS transpose reads (`ds_read_b64_tr_b16`) of four rows each.  In one such
+// read a group of 16 lanes supplies 16 addresses of 4 elements -- lane i: row r0 + (i >> 2), columns
+// m0 + 4 (i & 3) .. + 3 -- and lane i receives the elements [r0 .. r0 + 3][m0 + i].
 template <typename T>
-__device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const unsigned char* lds, int r0, int col) {
-  uint32_t w[4];
-#pragma unroll
-  for (int i = 0; i < 8; i += 2) {
-    const int ra = r0 + i, rb = r0 + i + 1;
-    const uint32_t lo = *reinterpret_cast<const uint16_t*>(
-        lds + ra * kFRowBytes + ((((col >> 3) ^ (ra & 15)) << 4) | ((col & 7) << 1)));
-    const uint32_t hi = *reinterpret_cast<const uint16_t*>(
-        lds + rb * kFRowBytes + ((((col >> 3) ^ (rb & 15)) << 4) | ((col & 7) << 1)));
-    w[i >> 1] = lo | (hi << 16);
-  }
-  return __builtin_bit_cast(typename Elem<T>::vec8, make_uint4(w[0], w[1], w[2], w[3]));
+__device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const unsigned char* lds, int k0, int col0,
+                                                                         int lane) {
+  const int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int ra = k0 + 8 * (lane >> 5) + ((lane >> 2) & 3);
+  const int rb = ra + 4;
+  const unsigned char* pa = lds + ra * kFRowBytes + ((((col >> 3) ^ (ra & 15)) << 4) | ((col & 7) << 1));
+  const unsigned char* pb = lds + rb * kFRowBytes + ((((col >> 3) ^ (rb & 15)) << 4) | ((col & 7) << 1));
+  struct {
+    short4_t lo, hi;
+  } v;
+  v.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(pa));
+  v.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(pb));
+  return __builtin_bit_cast(typename Elem<T>::vec8, v);
 }
 
-// s_waitcnt vmcnt(n) for a wave-uniform n in {0, 2, 4, 6, 8, 10} (the immediate must be a constant).
+// s_waitcnt vmcnt(n) for a wave-uniform n out of the values the ring below can ask for (the immediate
+// must be a constant); anything else waits for everything, which is always safe.
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
   switch (n) {
-    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
     case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
     case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
     case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+    case 18: asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); break;
+    case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
     default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
   }
 }
@@ -794,45 +803,55 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       }
       // Entries are packed at the front of a trip; the rows of absent ones are not fetched (loads
       // 2 e and 2 e + 1 of a wave belong to entry e), so a short trip moves proportionally less data.
+      // A short trip has small stages, so more of them fit the ring and more loads are in flight: a
+      // stage holds the rows of the present entries followed by the own rows.
       const int nent = min(4, list_n - li);
+      const int own_off = 32 * nent * kFRowBytes;
+      const int slot_bytes = own_off + kFOwnBytes;
+      const int ring = (nent >= 3) ? 3 : ((nent == 2) ? 5 : 7);  // slots of this size in the 120 KB ring
+      const int ahead = ring - 1;                              // stages in flight
       auto issue_stage = [&](int col0, int slot, bool with_own) {
-        const unsigned base = lds_base + slot * kFStageBytes;
+        const unsigned base = lds_base + slot * slot_bytes;
 #pragma unroll
         for (int q = 0; q < 8; ++q)
           if ((q >> 1) < nent) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
         if (with_own) {
 #pragma unroll
-          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + kFOtherBytes + (q * 4 + wave) * 1024);
+          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + own_off + (q * 4 + wave) * 1024);
         }
       };
 
-      // ---- logits^T of (entry of this wave) x (own rows): 10 loads per wave and stage, two stages ahead ----
+      // ---- logits^T of (entry of this wave) x (own rows): 2 nent + 2 loads per wave and stage -----------
       f32x16 s;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = 0.0f;
       const int last_col = (nstages - 1) * kFCols;
-      issue_stage(0, 0, true);
-      issue_stage(min(kFCols, last_col), 1, true);
+#pragma unroll 1
+      for (int j = 0; j < ahead; ++j) issue_stage(min(j * kFCols, last_col), j, true);
+      int slot = 0;  // st % ring
 #pragma unroll 1
       for (int st = 0; st < nstages; ++st) {
-        wait_vmcnt_upto(2 * nent + 2);  // all but the newest stage have landed
+        wait_vmcnt_upto((ahead - 1) * (2 * nent + 2));  // all but the newest stages have landed
         __syncthreads();                                   // ... for every wave; stage st - 1 is consumed
-        issue_stage(min((st + 2) * kFCols, last_col), (st + 2) % 3, true);
-        const unsigned char* so = smem + (st % 3) * kFStageBytes;
-        const unsigned char* sw = so + kFOtherBytes;
+        issue_stage(min((st + ahead) * kFCols, last_col), (slot == 0) ? ring - 1 : slot - 1, true);
+        const unsigned char* so = smem + slot * slot_bytes;
+        const unsigned char* sw = so + own_off;
+        slot = (slot + 1 == ring) ? 0 : slot + 1;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
           const auto fo = fstage_frag<T>(so, wave * 32 + l32, kk * 2 + half);
           const auto fw = fstage_frag<T>(sw, l32, kk * 2 + half);
-          s = IS_DE ? Elem<T>::mfma(fo, fw, s) : Elem<T>::mfma(fw, fo, s);
+          if (IS_DE) Elem<T>::mfma_vgpr(fo, fw, s);
+          else Elem<T>::mfma_vgpr(fw, fo, s);
         }
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the two unused prefetches
+      mfma_drain(s);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the unused prefetches
       __syncthreads();
-      // first two stages of the product phase, in flight during the epilogue
+      // first stages of the product phase, in flight during the epilogue
       const int last_chunk_col = d_begin + (nchunks - 1) * kFCols;
-      issue_stage(d_begin, 0, false);
-      issue_stage(min(d_begin + kFCols, last_chunk_col), 1, false);
+#pragma unroll 1
+      for (int j = 0; j < ahead; ++j) issue_stage(min(d_begin + j * kFCols, last_chunk_col), j, false);
 
       // ---- dz of this wave's 32 x 32 block (lane = token row, registers = classes) ----------------------------
       {
@@ -891,18 +910,21 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         bz[kk] = __builtin_bit_cast(typename Elem<T>::vec8, v);
       }
       if (product) {
+        int pslot = 0;  // ci % ring
 #pragma unroll
         for (int ci = 0; ci < kFMaxChunks; ++ci) {
           if (ci < nchunks) {
-            wait_vmcnt_upto(2 * nent);
+            wait_vmcnt_upto((ahead - 1) * 2 * nent);
             __syncthreads();
-            issue_stage(min(d_begin + (ci + 2) * kFCols, last_chunk_col), (ci + 2) % 3, false);
-            const unsigned char* so = smem + (ci % 3) * kFStageBytes;
+            issue_stage(min(d_begin + (ci + ahead) * kFCols, last_chunk_col), (pslot == 0) ? ring - 1 : pslot - 1, false);
+            const unsigned char* so = smem + pslot * slot_bytes;
+            pslot = (pslot + 1 == ring) ? 0 : pslot + 1;
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
               if ((mask >> (kk >> 1)) & 1u) {
-                const auto a = fstage_frag_transposed<T>(so, kk * 16 + half * 8, wave * 32 + l32);
-                acc[ci] = Elem<T>::mfma(a, bz[kk], acc[ci]);
+                const auto a = fstage_frag_transposed<T>(so, kk * 16, wave * 32, lane);
+                if (ci < 16) Elem<T>::mfma_agpr(a, bz[kk], acc[ci]);  // 16 chunks fill the 256 AGPRs
+                else Elem<T>::mfma_vgpr(a, bz[kk], acc[ci]);
               }
             }
           }
@@ -913,7 +935,57 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
     }
   }
 
-  if (write_out && touched) {
+  mfma_drain_all();  // the last product MFMAs, before anything else reads the accumulators
+  const bool out_fp32 = IS_DE ? (p.de_fp32 != 0) : (p.dc_fp32 != 0);
+  const bool out_vec = IS_DE ? (p.vec_e != 0) : (p.vec_c != 0);  // with the 8-element row strides of this kernel: 16-byte stores
+  if (write_out && touched && out_vec) {
+    // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
+    // are, one instruction would touch 32 rows with 16 bytes each.  Four chunks at a time go through
+    // LDS instead and leave as whole rows, 16 bytes per lane and 1 KB per row and instruction.
+    const int es = out_fp32 ? 4 : 2;
+    const int pitch = 4 * kFCols * es + 16;  // the odd 16 bytes spread the rows over the banks
+    unsigned char* out_base = static_cast<unsigned char*>(IS_DE ? p.d_e : p.d_c);
+#pragma unroll
+    for (int g = 0; g < (kFMaxChunks + 3) / 4; ++g) {
+      if (g * 4 < nchunks) {
+        __syncthreads();  // the ring is idle / the previous group has been read
+#pragma unroll
+        for (int cj = 0; cj < 4; ++cj) {
+          const int ci = g * 4 + cj;
+          if (ci < kFMaxChunks && ci < nchunks) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+              unsigned char* dst = smem + l32 * pitch + (cj * kFCols + wave * 32 + 8 * r4 + 4 * half) * es;
+              if (out_fp32) {
+                *reinterpret_cast<float4*>(dst) =
+                    make_float4(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 0], acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 1],
+                                acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 2], acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 3]);
+              } else {
+                uint2 pk;
+                pk.x = static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 0])) |
+                       (static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 1])) << 16);
+                pk.y = static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 2])) |
+                       (static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 3])) << 16);
+                *reinterpret_cast<uint2*>(dst) = pk;
+              }
+            }
+          }
+        }
+        __syncthreads();
+        const int ppr = min(4, nchunks - g * 4) * kFCols * es / 16;  // 16-byte pieces per row
+        for (int j = tid; j < 32 * ppr; j += kBwdThreads) {
+          const int row = j / ppr;
+          const int pc = j - row * ppr;
+          const int id = own_ids[row];
+          if (id >= 0) {
+            const uint4 v = *reinterpret_cast<const uint4*>(smem + row * pitch + pc * 16);
+            const int64_t off = (static_cast<int64_t>(id) * own_sr + d_begin + g * 4 * kFCols) * es + pc * 16;
+            *reinterpret_cast<uint4*>(out_base + off) = v;
+          }
+        }
+      }
+    }
+  } else if (write_out && touched) {
     const int id = own_ids[l32];
     if (id >= 0) {
 #pragma unroll

@@ -46,6 +46,17 @@ struct Elem<BF16> {
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // The same MFMA with the accumulator pinned to one register file: "a" = the accumulation registers
+  // (AGPRs), "v" = the ordinary ones.  For kernels whose accumulators outnumber the 256 AGPRs: the
+  // compiler places the results of all MFMA builtins of a function in one file and spills the excess,
+  // so such a kernel writes every one of its MFMAs this way and calls mfma_drain* before other kinds
+  // of instruction read the results.
+  static __device__ __forceinline__ void mfma_agpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_vgpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
     bf16x2_t v;
     v[0] = static_cast<__bf16>(lo);
@@ -67,6 +78,12 @@ struct Elem<F16> {
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma_agpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_vgpr(vec8 a, vec8 b, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
     f16x2_t v;
     v[0] = static_cast<_Float16>(lo);
@@ -74,6 +91,12 @@ struct Elem<F16> {
     __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<f16x2_t*>(addr), v);
   }
 };
+
+// The result of an MFMA written as inline assembly may be read by another kind of instruction only
+// after the matrix pipeline has drained (up to 18 wait states for a 32 x 32 block); the compiler
+// inserts those for its own MFMAs but cannot see into an asm statement.
+__device__ __forceinline__ void mfma_drain(f32x16& c) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(c)); }
+__device__ __forceinline__ void mfma_drain_all() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }
 
 // Add `val` to one 16-bit float in global memory through a compare-and-swap on the aligned
 // 32-bit word that contains it (used where a packed two-element atomic would be misaligned).
