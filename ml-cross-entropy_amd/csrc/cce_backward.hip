@@ -200,26 +200,46 @@ __device__ __forceinline__ float load_row_meta(const BwdParams& p, int64_t i, in
 
 // One 32 x 32 block of logits^T (lane = row `l32` of the group, registers = classes) -> dz.
 // Returns whether any |p - onehot| reaches eps.
-template <typename T>
-__device__ __forceinline__ bool block_epilogue(const BwdParams& p, f32x16& acc, const int* cid32, int half,
-                                               float lse2, float g, float h, int tgt) {
+template <typename T, bool CAP, bool HAS_BIAS>
+__device__ __forceinline__ bool block_epilogue_impl(const BwdParams& p, f32x16& acc, const int* cid32, int half,
+                                                    float lse2, float g, float h, int tgt) {
   bool big = false;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int cid = cid32[8 * (r >> 2) + 4 * half + (r & 3)];
-    float bias = 0.0f;
-    if (p.bias != nullptr && cid >= 0) bias = Elem<T>::to_float(p.bias[cid]);
-    float th;
-    const float s2 = softcap_log2(p.sc, acc[r] + bias, th);
+    float x = acc[r];
+    if (HAS_BIAS) x += (cid >= 0) ? Elem<T>::to_float(p.bias[cid]) : 0.0f;
+    float s2, damp = 1.0f;
+    if (CAP) {
+      const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
+      const float w = __builtin_amdgcn_rcpf(1.0f + t);
+      const float th = 1.0f - 2.0f * w;
+      s2 = p.sc.out_scale * th;
+      damp = 1.0f - th * th;
+    } else {
+      s2 = x * kLog2e;
+    }
     const float pr = (cid >= 0) ? __builtin_amdgcn_exp2f(s2 - lse2) : 0.0f;
     const bool hit = (cid >= 0) && (cid == tgt);
     const float f = pr - (hit ? 1.0f : 0.0f);
     big = big || (fabsf(f) >= p.filter_eps);
     float dz = pr * (g + h) - (hit ? g : 0.0f);
-    if (p.sc.on) dz *= (1.0f - th * th);
+    if (CAP) dz *= damp;
     acc[r] = dz;
   }
   return big;
+}
+
+// One uniform branch per block: each arm is straight-line code over the 16 values of a lane.
+template <typename T>
+__device__ __forceinline__ bool block_epilogue(const BwdParams& p, f32x16& acc, const int* cid32, int half,
+                                               float lse2, float g, float h, int tgt) {
+  if (p.bias != nullptr) {
+    if (p.sc.on) return block_epilogue_impl<T, true, true>(p, acc, cid32, half, lse2, g, h, tgt);
+    return block_epilogue_impl<T, false, true>(p, acc, cid32, half, lse2, g, h, tgt);
+  }
+  if (p.sc.on) return block_epilogue_impl<T, true, false>(p, acc, cid32, half, lse2, g, h, tgt);
+  return block_epilogue_impl<T, false, false>(p, acc, cid32, half, lse2, g, h, tgt);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -470,10 +490,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
               const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
               *reinterpret_cast<uint16_t*>(sDz + cls * 256 + ((((k >> 3) ^ (cls & 7)) << 4) | ((k & 7) << 1))) =
                   Elem<T>::from_float(s[r]);
-              float colsum = s[r];
+              if (p.d_bias != nullptr) {
+                float colsum = s[r];
 #pragma unroll
-              for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
-              if (l32 == 0) sDb[wave * 32 + cls] += colsum;  // one writer per slot: deterministic
+                for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
+                if (l32 == 0) sDb[wave * 32 + cls] += colsum;  // one writer per slot: deterministic
+              }
             }
           }
           if (lane == 0) atomicOr(&sMisc[1], 1 << wave);
@@ -623,6 +645,8 @@ __device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const u
 // must be a constant); anything else waits for everything, which is always safe.
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
   switch (n) {
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
     case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
     case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
     case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
@@ -735,6 +759,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       }
       if (wave == 0) {
         int n = 0;
+        uint32_t kept_word[4] = {0u, 0u, 0u, 0u};
         for (int base = 0; base < seg_n; base += 64) {
           if (IS_DE) {
             const int m = (base + lane < seg_n) ? sFlag[base + lane] : 0;
@@ -751,11 +776,17 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
               if ((m >> sb) & 1) sList[pos++] = (seg + base + lane) * 4 + sb;
             n += __shfl(incl, 63, 64);
           } else {
-            bool f = false;
-            if (base + lane < seg_n) {
-              const uint32_t w = p.kept_bits[static_cast<int64_t>(seg + base + lane) * p.bit_words + (own >> 5)];
-              f = ((w >> (own & 31)) & 1u) != 0u;
+            // four independent loads per lane, then four ballots: one round trip to memory per 256 row groups
+            if ((base & 255) == 0) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int u = base + j * 64 + lane;
+                uint32_t w = 0u;
+                if (u < seg_n) w = p.kept_bits[static_cast<int64_t>(seg + u) * p.bit_words + (own >> 5)];
+                kept_word[j] = w;
+              }
             }
+            const bool f = ((kept_word[(base >> 6) & 3] >> (own & 31)) & 1u) != 0u;
             const unsigned long long m = __ballot(f);
             if (f) sList[n + __popcll(m & ((1ull << lane) - 1ull))] = seg + base + lane;
             n += __popcll(m);
@@ -766,6 +797,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       __syncthreads();
     }
     const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
+    // A class group nothing survived for: its rows keep the zeros they came with.
+    if (!IS_DE && list_n == 0 && n_units <= seg_units) return;
 
     for (int li = 0; li < list_n; li += 4) {
       if (IS_DE) {
@@ -810,11 +843,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       const int slot_bytes = own_off + kFOwnBytes;
       const int ring = (nent >= 3) ? 3 : ((nent == 2) ? 5 : 7);  // slots of this size in the 120 KB ring
       const int ahead = ring - 1;                              // stages in flight
-      auto issue_stage = [&](int col0, int slot, bool with_own) {
+      auto issue_stage = [&](int col0, int slot, bool with_own, uint32_t entries) {
         const unsigned base = lds_base + slot * slot_bytes;
 #pragma unroll
         for (int q = 0; q < 8; ++q)
-          if ((q >> 1) < nent) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
+          if ((entries >> (q >> 1)) & 1u) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
         if (with_own) {
 #pragma unroll
           for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + own_off + (q * 4 + wave) * 1024);
@@ -826,14 +859,15 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = 0.0f;
       const int last_col = (nstages - 1) * kFCols;
+      const uint32_t present = (1u << nent) - 1u;
 #pragma unroll 1
-      for (int j = 0; j < ahead; ++j) issue_stage(min(j * kFCols, last_col), j, true);
+      for (int j = 0; j < ahead; ++j) issue_stage(min(j * kFCols, last_col), j, true, present);
       int slot = 0;  // st % ring
 #pragma unroll 1
       for (int st = 0; st < nstages; ++st) {
         wait_vmcnt_upto((ahead - 1) * (2 * nent + 2));  // all but the newest stages have landed
         __syncthreads();                                   // ... for every wave; stage st - 1 is consumed
-        issue_stage(min((st + ahead) * kFCols, last_col), (slot == 0) ? ring - 1 : slot - 1, true);
+        issue_stage(min((st + ahead) * kFCols, last_col), (slot == 0) ? ring - 1 : slot - 1, true, present);
         const unsigned char* so = smem + slot * slot_bytes;
         const unsigned char* sw = so + own_off;
         slot = (slot + 1 == ring) ? 0 : slot + 1;
@@ -848,10 +882,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       mfma_drain(s);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the unused prefetches
       __syncthreads();
-      // first stages of the product phase, in flight during the epilogue
       const int last_chunk_col = d_begin + (nchunks - 1) * kFCols;
-#pragma unroll 1
-      for (int j = 0; j < ahead; ++j) issue_stage(min(d_begin + j * kFCols, last_chunk_col), j, false);
 
       // ---- dz of this wave's 32 x 32 block (lane = token row, registers = classes) ----------------------------
       {
@@ -885,10 +916,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
               const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
               *reinterpret_cast<uint16_t*>(sDz + cls * 256 + ((((k >> 3) ^ (cls & 7)) << 4) | ((k & 7) << 1))) =
                   Elem<T>::from_float(s[r]);
-              float colsum = s[r];
+              if (p.d_bias != nullptr) {
+                float colsum = s[r];
 #pragma unroll
-              for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
-              if (l32 == 0) sDb[wave * 32 + cls] += colsum;
+                for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
+                if (l32 == 0) sDb[wave * 32 + cls] += colsum;
+              }
             }
           }
           if (lane == 0) atomicOr(&sMisc[1], 1 << wave);
@@ -910,13 +943,17 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         bz[kk] = __builtin_bit_cast(typename Elem<T>::vec8, v);
       }
       if (product) {
+        // Only the entries that are used are fetched again: the others would be read for nothing.
+        const int nused = __popc(mask);
+#pragma unroll 1
+        for (int j = 0; j < ahead; ++j) issue_stage(min(d_begin + j * kFCols, last_chunk_col), j, false, mask);
         int pslot = 0;  // ci % ring
 #pragma unroll
         for (int ci = 0; ci < kFMaxChunks; ++ci) {
           if (ci < nchunks) {
-            wait_vmcnt_upto((ahead - 1) * 2 * nent);
+            wait_vmcnt_upto((ahead - 1) * 2 * nused);
             __syncthreads();
-            issue_stage(min(d_begin + (ci + ahead) * kFCols, last_chunk_col), (pslot == 0) ? ring - 1 : pslot - 1, false);
+            issue_stage(min(d_begin + (ci + ahead) * kFCols, last_chunk_col), (pslot == 0) ? ring - 1 : pslot - 1, false, mask);
             const unsigned char* so = smem + pslot * slot_bytes;
             pslot = (pslot + 1 == ring) ? 0 : pslot + 1;
 #pragma unroll
@@ -937,8 +974,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 
   mfma_drain_all();  // the last product MFMAs, before anything else reads the accumulators
   const bool out_fp32 = IS_DE ? (p.de_fp32 != 0) : (p.dc_fp32 != 0);
-  const bool out_vec = IS_DE ? (p.vec_e != 0) : (p.vec_c != 0);  // with the 8-element row strides of this kernel: 16-byte stores
-  if (write_out && touched && out_vec) {
+  if (write_out && touched) {  // the launcher guarantees 16-byte aligned output rows
     // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
     // are, one instruction would touch 32 rows with 16 bytes each.  Four chunks at a time go through
     // LDS instead and leave as whole rows, 16 bytes per lane and 1 KB per row and instruction.
@@ -972,32 +1008,21 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
           }
         }
         __syncthreads();
-        const int ppr = min(4, nchunks - g * 4) * kFCols * es / 16;  // 16-byte pieces per row
-        for (int j = tid; j < 32 * ppr; j += kBwdThreads) {
-          const int row = j / ppr;
-          const int pc = j - row * ppr;
-          const int id = own_ids[row];
-          if (id >= 0) {
-            const uint4 v = *reinterpret_cast<const uint4*>(smem + row * pitch + pc * 16);
-            const int64_t off = (static_cast<int64_t>(id) * own_sr + d_begin + g * 4 * kFCols) * es + pc * 16;
-            *reinterpret_cast<uint4*>(out_base + off) = v;
-          }
-        }
-      }
-    }
-  } else if (write_out && touched) {
-    const int id = own_ids[l32];
-    if (id >= 0) {
-#pragma unroll
-      for (int ci = 0; ci < kFMaxChunks; ++ci) {
-        if (ci < nchunks) {
-          const int col0 = d_begin + ci * kFCols + wave * 32;
-          if (IS_DE)
-            store_rows<T>(acc[ci], p.d_e, p.de_fp32 != 0, p.vec_e != 0, static_cast<int64_t>(id) * p.stride_e, 1, col0,
-                          half, d_end);
-          else
-            store_rows<T>(acc[ci], p.d_c, p.dc_fp32 != 0, p.vec_c != 0, static_cast<int64_t>(id) * p.stride_cv,
-                          p.stride_cd, col0, half, d_end);
+        // 16-byte pieces per row: a multiple of 16, so one wave instruction stays inside one row and the
+        // 32 rows make at least two pieces per thread; two are read before either is stored.
+        const int ppr = min(4, nchunks - g * 4) * kFCols * es / 16;
+        for (int j = tid; j < 32 * ppr; j += 2 * kBwdThreads) {
+          const int ja = j, jb = j + kBwdThreads;
+          const int rowa = ja / ppr, rowb = jb / ppr;
+          const int pca = ja - rowa * ppr, pcb = jb - rowb * ppr;
+          const int ida = own_ids[rowa], idb = own_ids[rowb];
+          const uint4 va = *reinterpret_cast<const uint4*>(smem + rowa * pitch + pca * 16);
+          const uint4 vb = *reinterpret_cast<const uint4*>(smem + rowb * pitch + pcb * 16);
+          const int64_t col_bytes = static_cast<int64_t>(d_begin + g * 4 * kFCols) * es;
+          if (ida >= 0)
+            *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(ida) * own_sr * es + col_bytes + pca * 16) = va;
+          if (idb >= 0)
+            *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(idb) * own_sr * es + col_bytes + pcb * 16) = vb;
         }
       }
     }
@@ -1121,7 +1146,8 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
   const bool aligned = aligned16(e) && aligned16(c) && (d % 8 == 0) && (stride_e % 8 == 0) &&
                        (stride_cv % 8 == 0) && (stride_cd == 1);
   // The fast kernels want whole 128-column stages, also inside every slice of D.
-  const bool fast = aligned && (d % kFCols == 0);
+  // ... and they store whole 16-byte pieces of the output rows.
+  const bool fast = aligned && (d % kFCols == 0) && (d_e == nullptr || p.vec_e) && (d_c == nullptr || p.vec_c);
   hipError_t err;
 #define CCE_LAUNCH(KERN, LDS, GRID)                                                                 \
   do {                                                                                              \
