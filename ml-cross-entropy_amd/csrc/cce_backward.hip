@@ -476,10 +476,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
             for (int r4 = 0; r4 < 4; ++r4) {
               const int k = wave * 32 + 8 * r4 + 4 * half;
               uint2 pk;
-              pk.x = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 0])) |
-                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 1])) << 16);
-              pk.y = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 2])) |
-                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 3])) << 16);
+              pk.x = Elem<T>::pack2(s[r4 * 4 + 0], s[r4 * 4 + 1]);
+              pk.y = Elem<T>::pack2(s[r4 * 4 + 2], s[r4 * 4 + 3]);
               *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((k >> 3) ^ (l32 & 7)) << 4) | ((k & 7) << 1))) = pk;
             }
           } else {
@@ -903,10 +901,8 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
             for (int r4 = 0; r4 < 4; ++r4) {
               const int k = wave * 32 + 8 * r4 + 4 * half;
               uint2 pk;
-              pk.x = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 0])) |
-                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 1])) << 16);
-              pk.y = static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 2])) |
-                     (static_cast<uint32_t>(Elem<T>::from_float(s[r4 * 4 + 3])) << 16);
+              pk.x = Elem<T>::pack2(s[r4 * 4 + 0], s[r4 * 4 + 1]);
+              pk.y = Elem<T>::pack2(s[r4 * 4 + 2], s[r4 * 4 + 3]);
               *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((k >> 3) ^ (l32 & 7)) << 4) | ((k & 7) << 1))) = pk;
             }
           } else {
@@ -978,54 +974,57 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
     // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
     // are, one instruction would touch 32 rows with 16 bytes each.  Four chunks at a time go through
     // LDS instead and leave as whole rows, 16 bytes per lane and 1 KB per row and instruction.
-    const int es = out_fp32 ? 4 : 2;
-    const int pitch = 4 * kFCols * es + 16;  // the odd 16 bytes spread the rows over the banks
     unsigned char* out_base = static_cast<unsigned char*>(IS_DE ? p.d_e : p.d_c);
+    auto store_tile = [&](auto fp32_tag) {
+      constexpr bool FP32 = decltype(fp32_tag)::value;
+      constexpr int es = FP32 ? 4 : 2;
+      constexpr int pitch = 4 * kFCols * es + 16;  // the odd 16 bytes spread the rows over the banks
 #pragma unroll
-    for (int g = 0; g < (kFMaxChunks + 3) / 4; ++g) {
-      if (g * 4 < nchunks) {
-        __syncthreads();  // the ring is idle / the previous group has been read
+      for (int g = 0; g < (kFMaxChunks + 3) / 4; ++g) {
+        if (g * 4 < nchunks) {
+          __syncthreads();  // the ring is idle / the previous group has been read
 #pragma unroll
-        for (int cj = 0; cj < 4; ++cj) {
-          const int ci = g * 4 + cj;
-          if (ci < kFMaxChunks && ci < nchunks) {
+          for (int cj = 0; cj < 4; ++cj) {
+            constexpr int kLast = kFMaxChunks - 1;
+            const int ci = g * 4 + cj;
+            if (ci <= kLast && ci < nchunks) {
+              const f32x16& a = acc[ci <= kLast ? ci : kLast];
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-              unsigned char* dst = smem + l32 * pitch + (cj * kFCols + wave * 32 + 8 * r4 + 4 * half) * es;
-              if (out_fp32) {
-                *reinterpret_cast<float4*>(dst) =
-                    make_float4(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 0], acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 1],
-                                acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 2], acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 3]);
-              } else {
-                uint2 pk;
-                pk.x = static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 0])) |
-                       (static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 1])) << 16);
-                pk.y = static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 2])) |
-                       (static_cast<uint32_t>(Elem<T>::from_float(acc[ci < kFMaxChunks ? ci : 0][r4 * 4 + 3])) << 16);
-                *reinterpret_cast<uint2*>(dst) = pk;
+              for (int r4 = 0; r4 < 4; ++r4) {
+                unsigned char* dst = smem + l32 * pitch + (cj * kFCols + wave * 32 + 8 * r4 + 4 * half) * es;
+                if (FP32) {
+                  *reinterpret_cast<float4*>(dst) = make_float4(a[r4 * 4 + 0], a[r4 * 4 + 1], a[r4 * 4 + 2], a[r4 * 4 + 3]);
+                } else {
+                  uint2 pk;
+                  pk.x = Elem<T>::pack2(a[r4 * 4 + 0], a[r4 * 4 + 1]);
+                  pk.y = Elem<T>::pack2(a[r4 * 4 + 2], a[r4 * 4 + 3]);
+                  *reinterpret_cast<uint2*>(dst) = pk;
+                }
               }
             }
           }
-        }
-        __syncthreads();
-        // 16-byte pieces per row: a multiple of 16, so one wave instruction stays inside one row and the
-        // 32 rows make at least two pieces per thread; two are read before either is stored.
-        const int ppr = min(4, nchunks - g * 4) * kFCols * es / 16;
-        for (int j = tid; j < 32 * ppr; j += 2 * kBwdThreads) {
-          const int ja = j, jb = j + kBwdThreads;
-          const int rowa = ja / ppr, rowb = jb / ppr;
-          const int pca = ja - rowa * ppr, pcb = jb - rowb * ppr;
-          const int ida = own_ids[rowa], idb = own_ids[rowb];
-          const uint4 va = *reinterpret_cast<const uint4*>(smem + rowa * pitch + pca * 16);
-          const uint4 vb = *reinterpret_cast<const uint4*>(smem + rowb * pitch + pcb * 16);
-          const int64_t col_bytes = static_cast<int64_t>(d_begin + g * 4 * kFCols) * es;
-          if (ida >= 0)
-            *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(ida) * own_sr * es + col_bytes + pca * 16) = va;
-          if (idb >= 0)
-            *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(idb) * own_sr * es + col_bytes + pcb * 16) = vb;
+          __syncthreads();
+          // 16-byte pieces per row: a multiple of 16, so one wave instruction stays inside one row and the
+          // 32 rows make at least two pieces per thread; two are read before either is stored.
+          const int ppr = min(4, nchunks - g * 4) * kFCols * es / 16;
+          for (int j = tid; j < 32 * ppr; j += 2 * kBwdThreads) {
+            const int ja = j, jb = j + kBwdThreads;
+            const int rowa = ja / ppr, rowb = jb / ppr;
+            const int pca = ja - rowa * ppr, pcb = jb - rowb * ppr;
+            const int ida = own_ids[rowa], idb = own_ids[rowb];
+            const uint4 va = *reinterpret_cast<const uint4*>(smem + rowa * pitch + pca * 16);
+            const uint4 vb = *reinterpret_cast<const uint4*>(smem + rowb * pitch + pcb * 16);
+            const int64_t col_bytes = static_cast<int64_t>(d_begin + g * 4 * kFCols) * es;
+            if (ida >= 0)
+              *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(ida) * own_sr * es + col_bytes + pca * 16) = va;
+            if (idb >= 0)
+              *reinterpret_cast<uint4*>(out_base + static_cast<int64_t>(idb) * own_sr * es + col_bytes + pcb * 16) = vb;
+          }
         }
       }
-    }
+    };
+    if (out_fp32) store_tile(std::true_type{});
+    else store_tile(std::false_type{});
   }
   if (slice == 0) {
     if (IS_DE) {

@@ -43,6 +43,14 @@ struct Elem<BF16> {
     __bf16 h = static_cast<__bf16>(f);
     return __builtin_bit_cast(uint16_t, h);
   }
+  // two floats -> one packed pair (lo in the low half), one conversion instruction
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    float2_t f;
+    f[0] = lo;
+    f[1] = hi;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+  }
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -74,6 +82,13 @@ struct Elem<F16> {
   static __device__ __forceinline__ uint16_t from_float(float f) {
     _Float16 h = static_cast<_Float16>(f);
     return __builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    float2_t f;
+    f[0] = lo;
+    f[1] = hi;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_t));
   }
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
