@@ -43,9 +43,10 @@ extern "C" {
 #define CCE_STAT_ROWS 32
 #define CCE_STAT_COLS 128
 
-/* Number of uint64 slots in the backward counter block:
- * [0] tiles in the grid, [1] tiles whose logits were recomputed,
- * [2] tiles that ran the dE product, [3] tiles that ran the dC product. */
+/* Number of uint64 slots in the backward counter block, counted in sub-tiles of 32 rows x 32
+ * classes (the granularity of the gradient filter):
+ * [0] sub-tiles in the plane, [1] sub-tiles whose logits the dE pass recomputed,
+ * [2] sub-tiles that entered the dE product, [3] sub-tiles that entered the dC product. */
 #define CCE_NUM_COUNTERS 4
 
 /* Library ABI version (bumped when a signature below changes). */

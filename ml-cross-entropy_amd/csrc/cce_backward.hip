@@ -584,10 +584,17 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
 
 // ---------------------------------------------------------------------------------------------
 // Fast variant of the ownership kernel (16-byte aligned rows, unit column stride, D % 128 == 0):
-// the same algorithm with direct global -> LDS loads (no staging registers, no LDS stores) and a
-// ring of three 128-column stages, so that two stages of HBM / L2 latency are always in flight.
-// Both phases of a trip are latency-bound, not MFMA-bound, which is why the depth of the load
-// pipeline is what matters here.
+// the same algorithm with direct global -> LDS loads (no staging registers, no LDS stores) through a
+// ring of 128-column stages.  Both phases of a trip are bound by memory latency and gather
+// bandwidth, not by the MFMAs, so what matters is how much is in flight and how little is fetched:
+//   * a stage holds the rows of the entries that are present, then the own rows; a short trip has
+//     small stages, so 3 (3-4 entries), 5 (2) or 7 (1) of them fit the 120 KB ring;
+//   * the product phase fetches again only the entries whose dz is used;
+//   * the transposed product operand comes from the LDS transpose read, two per fragment;
+//   * all MFMAs are written as inline assembly with their accumulators pinned (16 chunks of the
+//     gradient in the 256 accumulation registers, the rest and the logits in ordinary registers):
+//     288 + 16 accumulator registers do not fit one file, and left alone the compiler spills;
+//   * the gradient tile leaves through LDS as whole rows, 1 KB per row and store instruction.
 //
 // Stage layout: 256-byte rows (128 columns), 16-byte chunks XOR-swizzled with (row & 15); one load
 // instruction of a wave fills 1 KB = 4 rows, lane l -> row (l >> 4), chunk slot (l & 15).  Other-side

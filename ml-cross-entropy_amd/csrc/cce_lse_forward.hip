@@ -1,8 +1,8 @@
 // cce_lse_forward: fused (E . C^T) -> soft-cap -> online log-sum-exp for gfx950.
 //
 // Work decomposition.  The (row-block, vocabulary) plane is cut into items: one item is a block
-// of 256 valid rows times a contiguous span of 256-wide vocabulary tiles.  A workgroup (4 waves,
-// 2 x 2, each wave 128 classes x 128 rows of accumulators) owns one item, walks its span tile by
+// of 256 valid rows times a contiguous span of 256-wide vocabulary tiles.  A workgroup (8 waves,
+// 2 x 4, each wave 128 classes x 64 rows of accumulators) owns one item, walks its span tile by
 // tile and keeps, per row, a running (max, sum-exp) pair in registers in the log2 domain.  At the
 // end the pairs of the two lane halves and of the two wave rows are merged and written as one
 // partial per (span, row); a second tiny kernel merges the spans.  No lock and no atomic is
