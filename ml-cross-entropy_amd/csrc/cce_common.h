@@ -577,26 +577,41 @@ struct DmaLogitTile {
     lds_dma16(ptr[q] + k0, lds_base + stage_off + blk * 1024);
   }
 
-  // The MFMAs of one step with loads [Q0, Q1) of a stage issued between them, one after every second
-  // MFMA.  Measured: a burst of all NQ loads right after the barrier backs up the address path, the
-  // waves that issue last fall a third of a stage behind and everybody waits for them at the next
-  // barrier; a steady trickle keeps the waves together.
+  // One 16-column step: the MFMAs on fragment set `cur`, and between them (one memory instruction per
+  // MFMA, so that this wave alone keeps the matrix pipeline fed while it issues them)
+  //   * the LDS reads of the next set `nxt` (step rkk of LDS stage rstage), ordered as the next step's
+  //     MFMAs will want them, and
+  //   * the direct-to-LDS loads [Q0, Q1) of a later stage, one after every second MFMA.
+  // Measured: a burst of all the loads of a stage right after the barrier backs up the address path,
+  // the waves that issue last fall a third of a stage behind and everybody waits for them at the next
+  // barrier; and a burst of fragment reads at the top of a step idles the matrix pipeline whenever both
+  // waves of a SIMD are in that burst together, which the barriers make the rule.
   template <int Q0, int Q1>
-  static __device__ __forceinline__ void mma_loads(f32x16 (&acc)[WV][WT], const Frags& f,
-                                                   const uint16_t* const (&ptr)[NQ], int k0, unsigned lds_base,
-                                                   int stage_off, int wave) {
+  static __device__ __forceinline__ void step(f32x16 (&acc)[WV][WT], const Frags& cur, Frags& nxt,
+                                              const unsigned char* lds, int rstage, int rkk, int coff0, int eoff0,
+                                              int sw, int half, const uint16_t* const (&ptr)[NQ], int k0,
+                                              unsigned lds_base, int lstage, int wave) {
     static_assert(Q1 - Q0 <= (WV * WT) / 2, "one load per two MFMAs");
+    static_assert(WV + WT <= WV * WT, "one fragment read per MFMA");
+    const int chunk = (((rkk * 2 + half) ^ sw) << 4);
+    const unsigned char* cb = lds + rstage + coff0 + chunk;
+    const unsigned char* eb = lds + rstage + eoff0 + chunk;
 #pragma unroll
     for (int vi = 0; vi < WV; ++vi)
 #pragma unroll
       for (int ti = 0; ti < WT; ++ti) {
-        acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
+        acc[vi][ti] = Elem<T>::mfma(cur.a[vi], cur.b[ti], acc[vi][ti]);
         const int idx = vi * WT + ti;
-        if ((idx & 1) && Q0 + idx / 2 < Q1) {
-          __builtin_amdgcn_sched_barrier(0);
-          issue_one(ptr, Q0 + idx / 2, k0, lds_base, stage_off, wave);
-          __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (idx == 0) {
+          nxt.a[0] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(cb));
+        } else if (idx <= WT) {
+          nxt.b[idx - 1] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(eb + (idx - 1) * 32 * kDmaRowBytes));
+        } else if (idx < WV + WT) {
+          nxt.a[idx - WT] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(cb + (idx - WT) * 32 * kDmaRowBytes));
         }
+        if ((idx & 1) && Q0 + idx / 2 < Q1) issue_one(ptr, Q0 + idx / 2, k0, lds_base, lstage, wave);
+        __builtin_amdgcn_sched_barrier(0);
       }
   }
 
@@ -641,36 +656,24 @@ struct DmaLogitTile {
     Frags fa = read_frags(lds, 0, 0, coff0, eoff0, sw, half);
     Frags fb;
 
-    // The scheduling fences pin "reads of the next step first, then this step's MFMAs": left alone,
-    // the compiler sinks every LDS read next to its use and the LDS latency is exposed.
+    // The scheduling fences inside step() pin the interleaving: left alone, the compiler sinks every
+    // LDS read next to its use and the LDS latency is exposed.
 #pragma unroll 1
     for (int s = 0; s < nk; ++s) {
       const int cur = (s & 1) * STAGE_BYTES;
       const int nxt = STAGE_BYTES - cur;
       const int k1 = min((s + 1) * kDmaBK, last);
       const int k2 = min((s + 2) * kDmaBK, last);
-      fb = read_frags(lds, cur, 1, coff0, eoff0, sw, half);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_loads<QA, QB>(acc, fa, ptr, k1, lds_base, nxt, wave);  // step 0
-      __builtin_amdgcn_sched_barrier(0);
-      fa = read_frags(lds, cur, 2, coff0, eoff0, sw, half);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_loads<QB, NQ>(acc, fb, ptr, k1, lds_base, nxt, wave);  // step 1
-      __builtin_amdgcn_sched_barrier(0);
-      fb = read_frags(lds, cur, 3, coff0, eoff0, sw, half);
-      __builtin_amdgcn_sched_barrier(0);
-      mma(acc, fa);  // step 2
-      __builtin_amdgcn_sched_barrier(0);
+      step<QA, QB>(acc, fa, fb, lds, cur, 1, coff0, eoff0, sw, half, ptr, k1, lds_base, nxt, wave);  // step 0
+      step<QB, NQ>(acc, fb, fa, lds, cur, 2, coff0, eoff0, sw, half, ptr, k1, lds_base, nxt, wave);  // step 1
+      step<NQ, NQ>(acc, fa, fb, lds, cur, 3, coff0, eoff0, sw, half, ptr, k1, lds_base, nxt, wave);  // step 2
       // Stage s + 1 (last loads issued two steps ago) has landed for this wave; after the barrier, for
       // every wave, and every wave holds its last fragments of stage s in registers: that LDS stage is
       // free and the first loads of stage s + 2 go into it.  A prefetch past the end re-reads the last
       // stage (never consumed), which keeps the loop free of branches.
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      fa = read_frags(lds, nxt, 0, coff0, eoff0, sw, half);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_loads<0, QA>(acc, fb, ptr, k2, lds_base, cur, wave);  // step 3
-      __builtin_amdgcn_sched_barrier(0);
+      step<0, QA>(acc, fb, fa, lds, nxt, 0, coff0, eoff0, sw, half, ptr, k2, lds_base, cur, wave);  // step 3
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch
     __syncthreads();  // every wave is done with the LDS (the last prefetch was awaited above)
