@@ -131,6 +131,32 @@ int cce_backward(const void* e, const void* c, const void* bias,
                  int64_t shift, int64_t target_offset,
                  float softcap, int dtype, void* stream);
 
+/* The logit gradient of one vocabulary chunk, written out, for the unfiltered backward.
+ *
+ * Restates the first half of the Triton backward body (cut_cross_entropy/cce_backward.py:
+ * logit recompute :170-188, softmax minus one-hot :196-207, d_out / d_lse scaling :238-248,
+ * soft-cap gradient :251, rounding to the input type :256) with the gradient filter off.  What the
+ * reference does next inside the same kernel -- the two products d_e += dz . c (:262-275) and
+ * d_c += dz^T . e (:289-302), through atomics -- is left to the caller: with every dz in play they
+ * are plain GEMMs (d_e[rows] += dz . c, d_c = dz^T . e[rows], d_bias = column sums of dz) on the
+ * [b, v] matrix this function fills, chunk of the vocabulary by chunk.
+ *
+ *   c, bias    the chunk's rows: v classes starting at the caller's offset
+ *   lse        [b] float, the LSE over the WHOLE vocabulary
+ *   dz         [b, ldz] in `dtype`, row i = valid row i (rows compacted through valids), ldz >= v
+ *   target_offset  first class of the chunk (plus the shard start, if any)
+ * Needs 16-byte aligned e, c, dz, unit stride_cd, row strides and ldz that are multiples of 8 and d a
+ * multiple of 64; anything else returns CCE_ERR_MISALIGNED and the caller uses cce_backward.
+ */
+int cce_backward_dz(const void* e, const void* c, const void* bias,
+                    const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                    const int32_t* valids, const int64_t* targets,
+                    void* dz, int64_t ldz,
+                    int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                    int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                    float grad_scale, int64_t shift, int64_t target_offset,
+                    float softcap, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,283 @@
+// cce_backward_dz: the gradient of the loss with respect to the logits of one vocabulary chunk,
+//     dz[i, j] = (p_ij (g_i + h_i) - [j == target_i] g_i) (1 - tanh^2)      p_ij = exp(s_ij - lse_i)
+// written to HBM in the input type, for the unfiltered ("exact") backward: with every entry of the
+// gradient in play the two products dE = dz . C and dC = dz^T . E are plain GEMMs, and the caller runs
+// them as such on the chunk.  The kernel is the forward kernel with another epilogue: same work
+// items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as whole rows
+// of 256 bytes per wave instruction after a transposition through LDS.
+#include "cce_common.h"
+
+namespace cce {
+
+struct DzParams {
+  const uint16_t* e;
+  const uint16_t* c;
+  const uint16_t* bias;
+  const int32_t* valids;
+  const float* lse;
+  const float* d_out;
+  const float* d_lse;
+  const int64_t* targets;
+  uint16_t* dz;
+  int64_t ldz;
+  int64_t n_rows, b, v, d;
+  int64_t stride_e, stride_cv;
+  int64_t shift, target_offset;
+  float grad_scale;
+  int d_out_is_scalar;
+  int nrb, nvt, nsplit, nitems, items_per_xcd;
+  Softcap sc;
+};
+
+constexpr int kDzWV = 4, kDzWT = 2, kDzNWV = 2, kDzNWT = 4;  // the forward kernel's wave tiling
+constexpr int kDzThreads = 64 * kDzNWV * kDzNWT;
+constexpr int kDzTile = 256;
+constexpr int kDzStagePitch = 128 * 2 + 16;  // one row of a wave's 32 x 128 block, padded against bank conflicts
+constexpr int kDzStageBytes = 32 * kDzStagePitch;
+
+template <typename T, bool GENERAL>
+__global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
+  using Fast = DmaLogitTile<T, kDzWV, kDzWT, kDzNWV, kDzNWT>;
+  static_assert(kDzStageBytes * kDzNWV * kDzNWT <= Fast::LDS_BYTES, "the staging blocks reuse the idle ring");
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_addend = reinterpret_cast<float*>(smem + Fast::LDS_BYTES);  // [2][256]
+
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  if (slot >= p.items_per_xcd) return;
+  const int item = xcd * p.items_per_xcd + slot;
+  if (item >= p.nitems) return;
+  const int rb = item / p.nsplit;
+  const int split = item % p.nsplit;
+  const int vt_begin = static_cast<int>((static_cast<int64_t>(p.nvt) * split) / p.nsplit);
+  const int vt_end = static_cast<int>((static_cast<int64_t>(p.nvt) * (split + 1)) / p.nsplit);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wv = wave / kDzNWT;
+  const int wt = wave % kDzNWT;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int64_t t0 = static_cast<int64_t>(rb) * kDzTile;
+
+  const uint16_t* fptr[Fast::NQ];
+#pragma unroll
+  for (int q = Fast::NQC; q < Fast::NQ; ++q) {
+    int64_t i = t0 + Fast::row_of(q, wave, lane);
+    i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
+    const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
+    fptr[q] = p.e + row * p.stride_e + Fast::chunk_elems(wave, lane);
+  }
+
+  // The two rows of this lane (one per 32-row column block): fixed for the whole item.
+  float r_lse2[kDzWT], r_g[kDzWT], r_h[kDzWT];
+  int r_tgt[kDzWT];
+#pragma unroll
+  for (int ti = 0; ti < kDzWT; ++ti) {
+    const int64_t i = t0 + wt * (32 * kDzWT) + ti * 32 + l32;
+    float lse2 = INFINITY, g = 0.0f, h = 0.0f;
+    int tgt = -1;
+    if (i < p.b) {
+      const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
+      lse2 = p.lse[i] * kLog2e;
+      const int64_t tpos = row + p.shift;
+      if (tpos < p.n_rows) {
+        const int64_t t = p.targets[tpos] - p.target_offset;
+        if (t >= 0 && t < p.v) tgt = static_cast<int>(t);
+        g = p.grad_scale * (p.d_out_is_scalar ? p.d_out[0] : p.d_out[tpos]);
+        if (p.d_lse != nullptr) h = p.d_lse[tpos];
+      }
+    }
+    r_lse2[ti] = lse2;
+    r_g[ti] = g;
+    r_h[ti] = h;
+    r_tgt[ti] = tgt;
+  }
+
+  unsigned char* stage = smem + wave * kDzStageBytes;
+
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int64_t v0 = static_cast<int64_t>(vt) * kDzTile;
+    float* addend = s_addend + (vt & 1) * kDzTile;
+    __syncthreads();  // every wave has left the staging blocks of the previous tile: the ring may be refilled
+#pragma unroll
+    for (int q = 0; q < Fast::NQC; ++q) {
+      int64_t vr = v0 + Fast::row_of(q, wave, lane);
+      vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked below
+      fptr[q] = p.c + vr * p.stride_cv + Fast::chunk_elems(wave, lane);
+    }
+    Fast::prefetch(fptr, smem, static_cast<int>(p.d));
+    if (GENERAL) {
+      if (tid < kDzTile) {  // published by the barriers of the main loop
+        const int64_t vg = v0 + tid;
+        float a = -INFINITY;
+        if (vg < p.v) a = (p.bias != nullptr) ? Elem<T>::to_float(p.bias[vg]) : 0.0f;
+        addend[tid] = a;
+      }
+    }
+    f32x16 acc[kDzWV][kDzWT];
+    Fast::run(acc, fptr, smem, static_cast<int>(p.d));
+
+    const int cls0 = static_cast<int>(v0) + wv * (32 * kDzWV);  // first class of this wave
+    const float* wave_addend = addend + wv * (32 * kDzWV);
+#pragma unroll
+    for (int ti = 0; ti < kDzWT; ++ti) {
+      const float lse2 = r_lse2[ti], g = r_g[ti], gh = r_g[ti] + r_h[ti];
+      const int tgt = r_tgt[ti];
+#pragma unroll
+      for (int vi = 0; vi < kDzWV; ++vi) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          float dzv[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int cl = vi * 32 + 8 * r4 + 4 * half + i;
+            float x = acc[vi][ti][r4 * 4 + i];
+            bool dead = false;
+            if (GENERAL) {
+              const float add = wave_addend[cl];
+              dead = (add == -INFINITY);
+              x = dead ? 0.0f : x + add;
+            }
+            float s2, damp = 1.0f;
+            if (p.sc.on) {
+              const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
+              const float w = __builtin_amdgcn_rcpf(1.0f + t);
+              const float th = 1.0f - 2.0f * w;
+              s2 = p.sc.out_scale * th;
+              damp = 1.0f - th * th;
+            } else {
+              s2 = x * kLog2e;
+            }
+            const float pr = __builtin_amdgcn_exp2f(s2 - lse2);
+            float dz = pr * gh - ((cls0 + cl == tgt) ? g : 0.0f);
+            dz *= damp;
+            dzv[i] = dead ? 0.0f : dz;
+          }
+          uint2 pk;
+          pk.x = Elem<T>::pack2(dzv[0], dzv[1]);
+          pk.y = Elem<T>::pack2(dzv[2], dzv[3]);
+          *reinterpret_cast<uint2*>(stage + l32 * kDzStagePitch + (vi * 32 + 8 * r4 + 4 * half) * 2) = pk;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is private to this wave: no barrier
+      // 32 rows x 256 bytes leave as 16-byte pieces: one instruction covers 4 rows of 256 contiguous bytes
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int j = lane + 64 * k;
+        const int row = j >> 4;
+        const int pc = j & 15;
+        const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kDzStagePitch + pc * 16);
+        const int64_t gi = t0 + wt * (32 * kDzWT) + ti * 32 + row;
+        const int64_t gcol = static_cast<int64_t>(cls0) + pc * 8;
+        if (gi < p.b) {
+          uint16_t* dst = p.dz + gi * p.ldz + gcol;
+          if (!GENERAL || gcol + 8 <= p.v) {
+            *reinterpret_cast<uint4*>(dst) = val;
+          } else {
+            const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (gcol + i < p.v) dst[i] = static_cast<uint16_t>(w[i >> 1] >> ((i & 1) * 16));
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block is staged
+    }
+  }
+}
+
+// Spans per row block: as in the forward kernel (enough items to fill the CUs, few beyond that).
+static int dz_choose_nsplit(int nrb, int nvt) {
+  const int num_cu = 256;
+  int best = 1;
+  double best_cost = 1e300;
+  const int max_split = nvt < 64 ? nvt : 64;
+  for (int s = 1; s <= max_split; ++s) {
+    const int64_t items = static_cast<int64_t>(nrb) * s;
+    const int64_t rounds = (items + num_cu - 1) / num_cu;
+    const int tiles_per_item = (nvt + s - 1) / s;
+    const double cost = static_cast<double>(rounds) * tiles_per_item + 0.02 * s;
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
+}  // namespace cce
+
+using namespace cce;
+
+extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
+                               const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                               const int32_t* valids, const int64_t* targets,
+                               void* dz, int64_t ldz,
+                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                               float grad_scale, int64_t shift, int64_t target_offset,
+                               float softcap, int dtype, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (b < 0 || v <= 0 || d <= 0 || n_rows < 0 || shift < 0 || ldz < v) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0) return CCE_OK;
+  if (e == nullptr || c == nullptr || lse == nullptr || d_out == nullptr || targets == nullptr || dz == nullptr)
+    return CCE_ERR_INVALID_ARGUMENT;
+  if (valids == nullptr && b > n_rows) return CCE_ERR_INVALID_ARGUMENT;
+  if (d > (1 << 30) || v > (int64_t(1) << 31) - 512) return CCE_ERR_INVALID_ARGUMENT;
+  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+  // direct-to-LDS main loop and 16-byte stores only
+  if (!aligned16(e) || !aligned16(c) || !aligned16(dz) || d % kDmaBK != 0 || stride_e % 8 != 0 ||
+      stride_cv % 8 != 0 || stride_cd != 1 || ldz % 8 != 0)
+    return CCE_ERR_MISALIGNED;
+
+  DzParams p;
+  p.e = static_cast<const uint16_t*>(e);
+  p.c = static_cast<const uint16_t*>(c);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.valids = valids;
+  p.lse = lse;
+  p.d_out = d_out;
+  p.d_lse = d_lse;
+  p.targets = targets;
+  p.dz = static_cast<uint16_t*>(dz);
+  p.ldz = ldz;
+  p.n_rows = n_rows;
+  p.b = b;
+  p.v = v;
+  p.d = d;
+  p.stride_e = stride_e;
+  p.stride_cv = stride_cv;
+  p.shift = shift;
+  p.target_offset = target_offset;
+  p.grad_scale = grad_scale;
+  p.d_out_is_scalar = d_out_is_scalar;
+  p.nrb = static_cast<int>((b + kDzTile - 1) / kDzTile);
+  p.nvt = static_cast<int>((v + kDzTile - 1) / kDzTile);
+  p.nsplit = dz_choose_nsplit(p.nrb, p.nvt);
+  p.nitems = p.nrb * p.nsplit;
+  p.items_per_xcd = (p.nitems + 7) / 8;
+  p.sc = make_softcap(softcap);
+
+  using FastB = DmaLogitTile<BF16, kDzWV, kDzWT, kDzNWV, kDzNWT>;
+  const int lds = FastB::LDS_BYTES + 2 * kDzTile * 4;
+  const bool general = (bias != nullptr) || (v % kDzTile != 0);
+  const int grid = p.items_per_xcd * 8;
+  hipError_t err;
+#define CCE_LAUNCH_DZ(TT, GE)                                                                     \
+  do {                                                                                            \
+    auto kern = dense_dz_kernel<TT, GE>;                                                          \
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+    if (err != hipSuccess) return status_from_hip(err);                                           \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kDzThreads), lds, stream, p);                       \
+  } while (0)
+  if (dtype == CCE_DTYPE_BF16) {
+    if (general) CCE_LAUNCH_DZ(BF16, true); else CCE_LAUNCH_DZ(BF16, false);
+  } else {
+    if (general) CCE_LAUNCH_DZ(F16, true); else CCE_LAUNCH_DZ(F16, false);
+  }
+#undef CCE_LAUNCH_DZ
+  return status_from_hip(hipGetLastError());
+}

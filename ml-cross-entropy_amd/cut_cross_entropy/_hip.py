@@ -44,6 +44,11 @@ _SIGNATURES = {
         [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]
         + [_i64] * 4 + [_i64] * 3 + [_f32, _f32, _i32, _i32, _i32, _i32, _i64, _i64, _f32, _i32, _ptr],
     ),
+    "cce_backward_dz": (
+        _i32,
+        [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _i64]
+        + [_i64] * 4 + [_i64] * 3 + [_f32, _i64, _i64, _f32, _i32, _ptr],
+    ),
 }
 
 

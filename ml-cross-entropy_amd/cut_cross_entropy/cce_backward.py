@@ -10,6 +10,82 @@ from cut_cross_entropy.cce_utils import filter_eps_or_none
 from cut_cross_entropy.utils import TensorInfo
 
 
+_DENSE_DZ_ELEMS = 1 << 26  # elements of one dz chunk (128 MB in a 16-bit type)
+
+
+def _mm_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``a @ b`` of 16-bit operands with the fp32 accumulator handed back unrounded."""
+    try:
+        return torch.mm(a, b, out_dtype=torch.float32)
+    except (TypeError, RuntimeError):  # a build without the mixed-precision GEMM: rounded per chunk
+        return torch.mm(a, b).to(torch.float32)
+
+
+def _dense_eligible(e, c, de, dc, dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
+    """The unfiltered backward runs as (dz kernel + library GEMMs) when nothing that is asked for is
+    filtered and the layout suits the direct-to-LDS kernel."""
+    if filter_eps_or_none(filter_eps) >= 0.0:
+        if (de is not None and filter_e_grad) or ((dc is not None or dbias is not None) and filter_c_grad):
+            return False
+    return (
+        e.size(1) % 64 == 0
+        and e.stride(0) % 8 == 0
+        and c.stride(1) == 1
+        and c.stride(0) % 8 == 0
+        and e.data_ptr() % 16 == 0
+        and c.data_ptr() % 16 == 0
+    )
+
+
+def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
+                    shift, target_offset, softcap):
+    """dE, dC, dBias of the unfiltered backward, one vocabulary chunk at a time: the kernel writes the
+    chunk's dz = d loss / d logits (never the logits), and the two products are library GEMMs
+    (reference: the products of cce_backward.py:262-302, there done with atomics inside the kernel).
+    dE is accumulated over the chunks in fp32; dC and dBias are complete per chunk."""
+    V, D = c.size(0), e.size(1)
+    vc = max(256, min(8192, (_DENSE_DZ_ELEMS // max(B, 1)) // 256 * 256))
+    vc = min(vc, (V + 7) // 8 * 8)
+    dz_buf = torch.empty((B * vc,), dtype=e.dtype, device=dev)
+    rows = valids.to(torch.int64) if valids is not None else None
+    e_rows = e if rows is None else e.index_select(0, rows)
+    de_acc = torch.zeros((B, D), dtype=torch.float32, device=dev) if de is not None else None
+    stream = _hip.current_stream_ptr(dev)
+    for v0 in range(0, V, vc):
+        n = min(vc, V - v0)
+        ldz = (n + 7) // 8 * 8
+        dz = dz_buf[: B * ldz].view(B, ldz)
+        c_chunk = c[v0 : v0 + n]
+        with torch.cuda.device(dev):
+            status = lib.cce_backward_dz(
+                e.data_ptr(), c_chunk.data_ptr(),
+                (bias.data_ptr() + v0 * bias.element_size()) if bias is not None else None,
+                lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
+                _hip.ptr(valids), targets.data_ptr(),
+                dz.data_ptr(), ldz,
+                e.size(0), B, n, D,
+                e.stride(0), c.stride(0), c.stride(1),
+                float(grad_scale), int(shift), int(target_offset) + v0,
+                float(softcap) if softcap is not None else 0.0, code, stream,
+            )
+        _hip.check(status, "cce_backward_dz")
+        dzv = dz[:, :n]
+        if de_acc is not None:
+            de_acc += _mm_fp32(dzv, c_chunk)
+        if dc is not None:
+            if dc.dtype == torch.float32:
+                dc[v0 : v0 + n] = _mm_fp32(dzv.t(), e_rows)
+            else:
+                torch.mm(dzv.t(), e_rows, out=dc[v0 : v0 + n])
+        if dbias is not None:
+            dbias[v0 : v0 + n] = dzv.sum(dim=0, dtype=torch.float32)
+    if de is not None:
+        if rows is None:
+            de.copy_(de_acc)
+        else:
+            de.index_copy_(0, rows, de_acc.to(de.dtype))
+
+
 def cce_backward_kernel(
     do: torch.Tensor,
     dlse: Optional[torch.Tensor],
@@ -111,7 +187,16 @@ def cce_backward_kernel(
         assert counters.dtype in (torch.int64, torch.uint64) and counters.numel() >= _hip.NUM_COUNTERS
         assert counters.is_contiguous() and counters.device == dev
 
-    if B > 0 and (de is not None or dc is not None or dbias is not None):
+    wanted = de is not None or dc is not None or dbias is not None
+    if B > 0 and wanted and _dense_eligible(e, c, de, dc, dbias, filter_eps, filter_e_grad, filter_c_grad):
+        _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
+                        shift, target_offset, softcap)
+        if counters is not None:  # every 32 x 32 sub-tile is recomputed and enters both products
+            tiles = ((B + 31) // 32) * ((c.size(0) + 31) // 32)
+            counters.view(torch.int64)[:4] += torch.tensor(
+                [tiles, tiles, tiles if de is not None else 0, tiles if dc is not None or dbias is not None else 0],
+                dtype=torch.int64, device=dev)
+    elif B > 0 and wanted:
         ws_bytes = lib.cce_backward_workspace_bytes(B, c.size(0), e.size(1))
         workspace = torch.empty((max(ws_bytes, 8) // 8 + 1,), dtype=torch.int64, device=dev)
         with torch.cuda.device(dev):

@@ -28,7 +28,8 @@ def _lib():
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for want in ("cce_version", "cce_error_string", "cce_tile_stat_elems", "cce_lse_forward_workspace_bytes",
-                 "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward"):
+                 "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward",
+                 "cce_backward_dz"):
         assert want in names
 
 

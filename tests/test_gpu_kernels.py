@@ -162,3 +162,74 @@ def test_backward_abi_exact(dtype, softcap, has_bias, with_dlse, shape):
     # without filtering every 32 x 32 sub-tile is recomputed and enters both products
     nt = ((valids.numel() + 31) // 32) * ((V + 31) // 32)
     assert counters.tolist() == [nt, nt, nt, nt]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("with_dlse", [False, True])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (255, 507, 64), (700, 1300, 192)])
+def test_backward_dz_abi(dtype, softcap, has_bias, with_dlse, shape):
+    """cce_backward_dz on two vocabulary chunks: the products of the dz it writes (formed here in
+    fp64) must be the closed-form dense gradients; rows past the valid ones and padding columns are
+    never written."""
+    from oracle import dense_lce
+
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=5, bias=has_bias, invalid_frac=0.2)
+    valids = dense_lce.build_flat_valids(t, IGNORE_INDEX, 0)
+    B = valids.numel()
+    g = torch.Generator().manual_seed(11)
+    d_out = torch.randn((N,), generator=g)
+    d_lse = torch.randn((N,), generator=g) * 0.1 if with_dlse else None
+    rows = valids.long()
+    lse = dense_lce.dense_lse(e[rows], c, bias, softcap, torch.float64)
+    gt = dense_lce.dense_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, torch.float64)
+    ref = autograd_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, dtype)
+
+    ed, cd, td, vd = e.to(dev), c.to(dev), t.to(dev), valids.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    lsed, dod = lse.float().to(dev), d_out.float().to(dev)
+    dld = d_lse.float().to(dev) if d_lse is not None else None
+    p = lambda x: x.data_ptr() if x is not None else None
+    split = (V // 2) // 8 * 8 + 8  # second chunk starts at a multiple of 8 that is not a tile boundary
+    dz_full = torch.zeros((B, V), dtype=torch.float64)
+    for v0, v1 in ((0, split), (split, V)):
+        n = v1 - v0
+        ldz = (n + 7) // 8 * 8 + 8  # one spare block of padding: must stay untouched
+        dz = torch.full((B + 3, ldz), 7.0, dtype=dtype, device=dev)
+        st = lib.cce_backward_dz(
+            p(ed), cd[v0:v1].data_ptr(), (bd.data_ptr() + 2 * v0) if bd is not None else None,
+            p(lsed), p(dod), 0, p(dld), p(vd), p(td), p(dz), ldz,
+            N, B, n, D, ed.stride(0), cd.stride(0), cd.stride(1),
+            0.5, 0, v0, softcap or 0.0, 0 if dtype == torch.bfloat16 else 1,
+            torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.cce_error_string(st)
+        torch.cuda.synchronize()
+        dzc = dz.cpu()
+        assert (dzc[B:] == 7.0).all() and (dzc[:, n:] == 7.0).all()
+        dz_full[:, v0:v1] = dzc[:B, :n].double()
+    de = torch.zeros((N, D), dtype=torch.float64)
+    de[rows] = dz_full @ c.double()
+    dc = dz_full.t() @ e[rows].double()
+    tol, rel = 2e-3, 1e-2
+    assert_no_worse(gt[0], ref[0], de, tol, "dE", rel)
+    assert_no_worse(gt[1], ref[1], dc, tol, "dC", rel)
+    if has_bias:
+        assert_no_worse(gt[2], ref[2], dz_full.sum(0), tol, "dBias", rel)
+
+
+def test_backward_dz_rejects_layouts_it_cannot_stream():
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    e = torch.zeros((64, 72), dtype=torch.bfloat16, device=dev)  # D % 64 != 0
+    c = torch.zeros((128, 72), dtype=torch.bfloat16, device=dev)
+    lse = torch.zeros((64,), device=dev)
+    t = torch.zeros((64,), dtype=torch.int64, device=dev)
+    dz = torch.zeros((64, 128), dtype=torch.bfloat16, device=dev)
+    st = lib.cce_backward_dz(e.data_ptr(), c.data_ptr(), None, lse.data_ptr(), lse.data_ptr(), 0, None, None,
+                             t.data_ptr(), dz.data_ptr(), 128, 64, 64, 128, 72, 72, 72, 1, 1.0, 0, 0, 0.0, 0,
+                             torch.cuda.current_stream().cuda_stream)
+    assert st == 10004  # CCE_ERR_MISALIGNED

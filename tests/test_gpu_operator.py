@@ -170,3 +170,37 @@ def test_deterministic_forward():
     a = linear_cross_entropy(e, c, t, reduction="none")
     b = linear_cross_entropy(e, c, t, reduction="none")
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("impl", ["cce_exact", "cce_kahan_full_c_full_e"])
+@pytest.mark.parametrize("with_valids", [False, True])
+def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids):
+    """Aligned shapes with the filter off run the dz kernel + GEMM backward (and still match the oracle);
+    a hidden size the direct-to-LDS kernel cannot stream falls back to the ownership kernels."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    calls = []
+    real = bw._dense_backward
+    monkeypatch.setattr(bw, "_dense_backward", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+
+    def run(D):
+        e, c, t, _ = make_inputs(384, 1100, D, torch.bfloat16, seed=2, invalid_frac=0.25 if with_valids else 0.0)
+        ed = e.cuda().requires_grad_(True)
+        cd = c.cuda().requires_grad_(True)
+        loss = linear_cross_entropy(ed, cd, t.cuda(), softcap=25.0, impl=impl, shift=1 if with_valids else 0)
+        loss.backward()
+        e64 = e.double().requires_grad_(True)
+        c64 = c.double().requires_grad_(True)
+        want, _ = dense_lce.dense_linear_cross_entropy(e64, c64, t, softcap=25.0, shift=1 if with_valids else 0)
+        want.backward()
+        assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+        scale = 1.0 / 384
+        assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=2e-2 * scale, rtol=2e-2)
+        assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=2e-2 * scale, rtol=2e-2)
+
+    run(128)
+    assert len(calls) == 1
+    run(72)
+    assert len(calls) == 1
