@@ -21,11 +21,11 @@ def _mm_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         return torch.mm(a, b).to(torch.float32)
 
 
-def _dense_eligible(e, c, de, dc, dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
+def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
     """The unfiltered backward runs as (dz kernel + library GEMMs) when nothing that is asked for is
     filtered and the layout suits the direct-to-LDS kernel."""
     if filter_eps_or_none(filter_eps) >= 0.0:
-        if (de is not None and filter_e_grad) or ((dc is not None or dbias is not None) and filter_c_grad):
+        if (want_de and filter_e_grad) or ((want_dc or want_dbias) and filter_c_grad):
             return False
     return (
         e.size(1) % 64 == 0
@@ -155,6 +155,13 @@ def cce_backward_kernel(
 
     de_dtype = torch.float32 if accum_e_fp32 else e.dtype
     dc_dtype = torch.float32 if accum_c_fp32 else c.dtype
+    dense = _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad,
+                            bias is not None and bias_info is not None and bias_info.requires_grad,
+                            filter_eps, filter_e_grad, filter_c_grad)
+    if dense:
+        # every GEMM of the dense path accumulates in fp32 internally and each output element is written
+        # once (dC, dBias) or summed in a separate fp32 buffer (dE): no fp32 gradient buffers are needed
+        de_dtype, dc_dtype = e_info.dtype, c_info.dtype
     de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
     dc = torch.zeros_like(c, dtype=dc_dtype) if c_info.requires_grad else None
     dbias = None
@@ -188,7 +195,7 @@ def cce_backward_kernel(
         assert counters.is_contiguous() and counters.device == dev
 
     wanted = de is not None or dc is not None or dbias is not None
-    if B > 0 and wanted and _dense_eligible(e, c, de, dc, dbias, filter_eps, filter_e_grad, filter_c_grad):
+    if B > 0 and wanted and dense:
         _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
                         shift, target_offset, softcap)
         if counters is not None:  # every 32 x 32 sub-tile is recomputed and enters both products
