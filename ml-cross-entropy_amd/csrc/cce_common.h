@@ -680,6 +680,32 @@ struct DmaLogitTile {
   }
 };
 
+// Vocabulary spans per row block for the kernels that cut the (row block, vocabulary) plane into
+// items of one row block x one span of tiles.  Two things are weighed: the rounds of 256 workgroups
+// the items make, and the L2 traffic of the 32 workgroups that run on one XCD at a time, which cover
+// 32 / s row blocks (one E block each) times s spans (one stream of C tiles each): s + 32 / s streams,
+// least for s = 4 .. 8.  The weight 0.165 is fitted to measurements at E [65536, 3584] x C [152064, 3584]
+// (1, 2, 4, 8, 16 spans: 70.8, 62.5, 53.9, 56.8, 59.4 ms).
+inline int choose_span_count(int nrb, int nvt) {
+  const int num_cu = 256;
+  int best = 1;
+  double best_cost = 1e300;
+  const int max_split = nvt < 64 ? nvt : 64;
+  for (int s = 1; s <= max_split; ++s) {
+    const int64_t items = static_cast<int64_t>(nrb) * s;
+    const int64_t rounds = (items + num_cu - 1) / num_cu;
+    const int tiles_per_item = (nvt + s - 1) / s;
+    const double streams = (s <= 32) ? s + 32.0 / s : s + 1.0;
+    const double traffic = 1.0 + 0.165 * (streams / 11.3137 - 1.0);
+    const double cost = static_cast<double>(rounds) * tiles_per_item * traffic + 0.02 * s;
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
 inline int status_from_hip(hipError_t e) { return e == hipSuccess ? CCE_OK : static_cast<int>(e); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

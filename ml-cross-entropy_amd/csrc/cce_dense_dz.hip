@@ -188,25 +188,6 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
   }
 }
 
-// Spans per row block: as in the forward kernel (enough items to fill the CUs, few beyond that).
-static int dz_choose_nsplit(int nrb, int nvt) {
-  const int num_cu = 256;
-  int best = 1;
-  double best_cost = 1e300;
-  const int max_split = nvt < 64 ? nvt : 64;
-  for (int s = 1; s <= max_split; ++s) {
-    const int64_t items = static_cast<int64_t>(nrb) * s;
-    const int64_t rounds = (items + num_cu - 1) / num_cu;
-    const int tiles_per_item = (nvt + s - 1) / s;
-    const double cost = static_cast<double>(rounds) * tiles_per_item + 0.02 * s;
-    if (cost < best_cost - 1e-9) {
-      best_cost = cost;
-      best = s;
-    }
-  }
-  return best;
-}
-
 }  // namespace cce
 
 using namespace cce;
@@ -255,7 +236,7 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
   p.d_out_is_scalar = d_out_is_scalar;
   p.nrb = static_cast<int>((b + kDzTile - 1) / kDzTile);
   p.nvt = static_cast<int>((v + kDzTile - 1) / kDzTile);
-  p.nsplit = dz_choose_nsplit(p.nrb, p.nvt);
+  p.nsplit = choose_span_count(p.nrb, p.nvt);
   p.nitems = p.nrb * p.nsplit;
   p.items_per_xcd = (p.nitems + 7) / 8;
   p.sc = make_softcap(softcap);

@@ -299,25 +299,7 @@ __global__ void fill_zero_kernel(float* p, int64_t n) {
   if (i < n) p[i] = 0.0f;
 }
 
-// Spans per row block: enough items to fill the CUs, as few as possible beyond that
-// (each extra span re-reads the E block's share of L2 and writes one more partial).
-static int choose_nsplit(int nrb, int nvt) {
-  const int num_cu = 256;
-  int best = 1;
-  double best_cost = 1e300;
-  const int max_split = nvt < 64 ? nvt : 64;
-  for (int s = 1; s <= max_split; ++s) {
-    const int64_t items = static_cast<int64_t>(nrb) * s;
-    const int64_t rounds = (items + num_cu - 1) / num_cu;
-    const int tiles_per_item = (nvt + s - 1) / s;
-    const double cost = static_cast<double>(rounds) * tiles_per_item + 0.02 * s;
-    if (cost < best_cost - 1e-9) {
-      best_cost = cost;
-      best = s;
-    }
-  }
-  return best;
-}
+static int choose_nsplit(int nrb, int nvt) { return choose_span_count(nrb, nvt); }
 
 template <typename T>
 static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipStream_t stream) {
