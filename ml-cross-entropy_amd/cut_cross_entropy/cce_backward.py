@@ -12,6 +12,25 @@ from cut_cross_entropy.utils import TensorInfo
 
 _DENSE_DZ_ELEMS = 1 << 26  # elements of one dz chunk (128 MB in a 16-bit type)
 
+# With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path
+# pays for the whole plane once: measured on MI355X the two cross where about one 128-class cell in
+# seven can hold a probability above filter_eps.  Above this fraction (read off the forward pass's
+# tile statistic, one small reduction and one host read) the backward is run unfiltered; an unfiltered
+# gradient is the exact one, so nothing is lost.  None switches the test off.
+DENSE_WHEN_FLAGGED_ABOVE = 0.12
+
+
+def _flagged_fraction(tile_max, lse, B, V, filter_eps) -> float:
+    """Fraction of the 32-row x 128-class cells whose bound exp(max logit - min lse) reaches filter_eps."""
+    import math
+
+    ntg, nvc = (B + 31) // 32, (V + _hip.STAT_COLS - 1) // _hip.STAT_COLS
+    lse_pad = torch.full((ntg * 32,), float("inf"), dtype=torch.float32, device=lse.device)
+    lse_pad[:B] = lse
+    lse_min = lse_pad.view(ntg, 32).min(dim=1).values
+    bound = tile_max.view(ntg, nvc) - lse_min[:, None]
+    return float((bound >= math.log(filter_eps) - 0.01).float().mean().item())
+
 
 def _mm_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     """``a @ b`` of 16-bit operands with the fp32 accumulator handed back unrounded."""
@@ -158,6 +177,12 @@ def cce_backward_kernel(
     dense = _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad,
                             bias is not None and bias_info is not None and bias_info.requires_grad,
                             filter_eps, filter_e_grad, filter_c_grad)
+    if (not dense and DENSE_WHEN_FLAGGED_ABOVE is not None and tile_max is not None and filter_eps is not None
+            and filter_eps > 0 and lse.numel() > 0
+            and _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad, False, None, False, False)):
+        n_valid = valids.size(0) if valids is not None else e.size(0)
+        dense = _flagged_fraction(tile_max, lse.to(torch.float32), n_valid, c.size(0), float(filter_eps)) \
+            > DENSE_WHEN_FLAGGED_ABOVE
     if dense:
         # every GEMM of the dense path accumulates in fp32 internally and each output element is written
         # once (dC, dBias) or summed in a separate fp32 buffer (dE): no fp32 gradient buffers are needed

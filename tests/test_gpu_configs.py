@@ -94,10 +94,13 @@ def test_config1_small_reference_run():
     assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
     valids = _build_flat_valids(td, IGNORE_INDEX, 0)
     d_out = torch.full((N,), 1.0 / valids.numel(), device=DEV)
+    # "allowing for filter-skipped entries": the filtered oracle when the sparse kernels ran, the exact one
+    # when the backward chose to run unfiltered (it does when most cells could hold a probability >= eps)
     _, de, dc, _ = _oracle_on_gpu(e.to(DEV), c.to(DEV), td.clamp_min(0), valids, d_out, None, None,
                                   filter_eps=2.0**-12)
-    assert _rel_err(ed.grad, de) <= 1e-2
-    assert _rel_err(cd.grad, dc) <= 1e-2
+    _, de_x, dc_x, _ = _oracle_on_gpu(e.to(DEV), c.to(DEV), td.clamp_min(0), valids, d_out, None, None)
+    assert min(_rel_err(ed.grad, de), _rel_err(ed.grad, de_x)) <= 1e-2
+    assert min(_rel_err(cd.grad, dc), _rel_err(cd.grad, dc_x)) <= 1e-2
     ign = t == IGNORE_INDEX
     assert (ed.grad.cpu()[ign] == 0).all()  # bit-exact masking
     # and the unfiltered preset against the unfiltered oracle

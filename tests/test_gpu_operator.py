@@ -204,3 +204,39 @@ def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids
     assert len(calls) == 1
     run(72)
     assert len(calls) == 1
+
+
+def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
+    """Near-uniform soft-max over few classes: every cell's bound exp(max logit - min lse) is above
+    filter_eps, so the backward runs unfiltered (and is then exact); with the switch off the
+    ownership kernels run.  Peaked soft-max over many classes: the sparse kernels stay."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    calls = []
+    real = bw._dense_backward
+    monkeypatch.setattr(bw, "_dense_backward", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+
+    e, c, t, _ = make_inputs(512, 2048, 128, torch.bfloat16, seed=4, planted=False, c_std=0.05)
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    assert len(calls) == 1
+    e64, c64 = e.double().requires_grad_(True), c.double().requires_grad_(True)
+    dense_lce.dense_linear_cross_entropy(e64, c64, t)[0].backward()
+    assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=2e-2 / 512, rtol=2e-2)
+    assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=2e-2 / 512, rtol=2e-2)
+
+    monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", None)
+    ed.grad = cd.grad = None
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    assert len(calls) == 1
+
+    monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", 0.12)
+    g = torch.Generator().manual_seed(1)
+    c2 = (torch.randn((65536, 128), generator=g) * 0.5).to(torch.bfloat16)  # 512 cells per row group, <= 32 hold a target
+    t2 = torch.randint(0, 65536, (512,), generator=g)
+    e2 = (c2[t2].float() * 4).to(torch.bfloat16)  # each row points at its own class: a peaked soft-max
+    ed2, cd2 = e2.cuda().requires_grad_(True), c2.cuda().requires_grad_(True)
+    linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
+    assert len(calls) == 1
