@@ -41,7 +41,7 @@ extern "C" {
 
 /* Granularity of the forward tile statistic (rows x vocabulary entries per cell). */
 #define CCE_STAT_ROWS 32
-#define CCE_STAT_COLS 128
+#define CCE_STAT_COLS 32
 
 /* Number of uint64 slots in the backward counter block, counted in sub-tiles of 32 rows x 32
  * classes (the granularity of the gradient filter):

@@ -345,8 +345,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
       if (IS_DE) {
         // a cell whose bound reaches eps needs all four sub-blocks; otherwise only those holding a target
         for (int j = tid; j < seg_n; j += kBwdThreads) {
-          const float cell = p.tile_max[static_cast<int64_t>(own) * p.stat_cols + seg + j];
-          sFlag[j] = (cell - min_lse >= p.log_eps) ? 0xF : 0;
+          // one bound per 32-class sub-block: exp(max logit - min lse of the 32 rows) against eps
+          const float* cell = p.tile_max + static_cast<int64_t>(own) * p.stat_cols + static_cast<int64_t>(seg + j) * 4;
+          const int nsb = min(4, p.stat_cols - (seg + j) * 4);
+          int m = 0;
+#pragma unroll
+          for (int sb = 0; sb < 4; ++sb)
+            if (sb < nsb && cell[sb] - min_lse >= p.log_eps) m |= 1 << sb;
+          sFlag[j] = static_cast<unsigned char>(m);
         }
         __syncthreads();
         if (tid < 32) {
@@ -748,8 +754,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
     if (use_list) {
       if (IS_DE) {
         for (int j = tid; j < seg_n; j += kBwdThreads) {
-          const float cell = p.tile_max[static_cast<int64_t>(own) * p.stat_cols + seg + j];
-          sFlag[j] = (cell - min_lse >= p.log_eps) ? 0xF : 0;
+          // one bound per 32-class sub-block: exp(max logit - min lse of the 32 rows) against eps
+          const float* cell = p.tile_max + static_cast<int64_t>(own) * p.stat_cols + static_cast<int64_t>(seg + j) * 4;
+          const int nsb = min(4, p.stat_cols - (seg + j) * 4);
+          int m = 0;
+#pragma unroll
+          for (int sb = 0; sb < 4; ++sb)
+            if (sb < nsb && cell[sb] - min_lse >= p.log_eps) m |= 1 << sb;
+          sFlag[j] = static_cast<unsigned char>(m);
         }
         __syncthreads();
         if (tid < 32) {

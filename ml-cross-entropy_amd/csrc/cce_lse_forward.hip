@@ -37,7 +37,7 @@ constexpr int kFwdWV = 4, kFwdWT = 2, kFwdNWV = 2, kFwdNWT = 4;
 constexpr int kFwdThreads = 64 * kFwdNWV * kFwdNWT;
 constexpr int kFwdTile = 256;
 static_assert(32 * kFwdWV * kFwdNWV == kFwdTile && 32 * kFwdWT * kFwdNWT == kFwdTile, "tile is 256 x 256");
-static_assert(32 * kFwdWV == CCE_STAT_COLS, "one statistic cell per (wave, 32-row block)");
+static_assert(CCE_STAT_COLS == 32 && CCE_STAT_ROWS == 32, "one statistic cell per 32 x 32 accumulator block");
 
 constexpr int kFwdBiasBytes = 2 * 256 * 4;  // two tiles' worth of per-class addends (double-buffered)
 
@@ -47,10 +47,12 @@ constexpr int kFwdBiasBytes = 2 * 256 * 4;  // two tiles' worth of per-class add
 // The plain variant is straight-line code with no loads.
 template <bool GENERAL, bool CAP>
 __device__ __forceinline__ float column_block_logits_impl(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
-                                                          const float* addend, int half, float (&s2)[kFwdWV][16]) {
+                                                          const float* addend, int half, float (&s2)[kFwdWV][16],
+                                                          float (&bm)[kFwdWV]) {
   float tm = -INFINITY;
 #pragma unroll
   for (int vi = 0; vi < kFwdWV; ++vi) {
+    bm[vi] = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       float x = acc[vi][ti][r];
@@ -70,8 +72,9 @@ __device__ __forceinline__ float column_block_logits_impl(const Softcap& sc, con
         y = x * kLog2e;
       }
       s2[vi][r] = dead ? -INFINITY : y;
-      tm = fmaxf(tm, s2[vi][r]);
+      bm[vi] = fmaxf(bm[vi], s2[vi][r]);
     }
+    tm = fmaxf(tm, bm[vi]);
   }
   return tm;
 }
@@ -80,9 +83,10 @@ __device__ __forceinline__ float column_block_logits_impl(const Softcap& sc, con
 // independent exp2 / rcp chains of different values overlap.
 template <bool GENERAL>
 __device__ __forceinline__ float column_block_logits(const Softcap& sc, const f32x16 (&acc)[kFwdWV][kFwdWT], int ti,
-                                                     const float* addend, int half, float (&s2)[kFwdWV][16]) {
-  if (sc.on) return column_block_logits_impl<GENERAL, true>(sc, acc, ti, addend, half, s2);
-  return column_block_logits_impl<GENERAL, false>(sc, acc, ti, addend, half, s2);
+                                                     const float* addend, int half, float (&s2)[kFwdWV][16],
+                                                     float (&bm)[kFwdWV]) {
+  if (sc.on) return column_block_logits_impl<GENERAL, true>(sc, acc, ti, addend, half, s2, bm);
+  return column_block_logits_impl<GENERAL, false>(sc, acc, ti, addend, half, s2, bm);
 }
 
 // Kernel variants:
@@ -205,7 +209,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
     for (int ti = 0; ti < kFwdWT; ++ti) {
       __builtin_amdgcn_sched_barrier(0);  // keep each column block's register use to itself
       float s2[kFwdWV][16];
-      const float tm = column_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, half, s2);
+      float bm[kFwdWV];  // this lane's maximum in each of the four 32-class blocks
+      const float tm = column_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, half, s2, bm);
       if (WANT_LA) {
         const float ok = (t0 + wt * (32 * kFwdWT) + ti * 32 + l32 < p.b) ? 1.0f : 0.0f;
 #pragma unroll
@@ -215,12 +220,18 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
       }
 
       if (p.tile_max != nullptr) {
-        // max over the 32 rows x 128 classes of this (wave, ti) cell
-        const float cell = wave_max(tm);
+        // max over the 32 rows x 32 classes of each accumulator block of this (wave, ti)
         const int64_t srow = (t0 + wt * (32 * kFwdWT) + ti * 32) / CCE_STAT_ROWS;
         const int64_t scol = vw0 / CCE_STAT_COLS;
-        if (lane == 0 && (t0 + wt * (32 * kFwdWT) + ti * 32) < p.b && vw0 < p.v)
-          p.tile_max[srow * p.stat_cols + scol] = cell * kLn2;
+        float cell[kFwdWV];
+#pragma unroll
+        for (int vi = 0; vi < kFwdWV; ++vi) cell[vi] = wave_max(bm[vi]);
+        if (lane < kFwdWV && (t0 + wt * (32 * kFwdWT) + ti * 32) < p.b && vw0 + lane * 32 < p.v) {
+          float mine = cell[0];
+#pragma unroll
+          for (int vi = 1; vi < kFwdWV; ++vi) mine = (lane == vi) ? cell[vi] : mine;
+          p.tile_max[srow * p.stat_cols + scol + lane] = mine * kLn2;
+        }
       }
 
       const float mn = fmaxf(m2[ti], tm);

@@ -16,10 +16,10 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
 STAT_ROWS = 32
-STAT_COLS = 128
+STAT_COLS = 32
 NUM_COUNTERS = 4
 
 _i64, _i32, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p

@@ -19,7 +19,7 @@ def lse_forward(
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """Returns ``(lse[B] fp32, logit_avg[V] fp32 | None, tile_max | None)``.
 
-    ``tile_max`` holds the largest soft-capped logit of every 32-row x 128-class cell;
+    ``tile_max`` holds the largest soft-capped logit of every 32-row x 32-class cell;
     the backward uses it to drop tiles without recomputing them.
     """
     assert e.ndim == 2 and c.ndim == 2

@@ -53,8 +53,8 @@ def test_host_only_queries():
     assert lib.cce_error_string(0) == b"success"
     assert b"workspace" in lib.cce_error_string(10003)
     # ceil(8192 / 32) * ceil(256000 / 128)
-    assert lib.cce_tile_stat_elems(8192, 256000) == 256 * 2000
-    assert lib.cce_tile_stat_elems(33, 129) == 2 * 2
+    assert lib.cce_tile_stat_elems(8192, 256000) == 256 * 8000
+    assert lib.cce_tile_stat_elems(33, 129) == 2 * 5
     assert lib.cce_tile_stat_elems(0, 100) == 0
     ws = lib.cce_lse_forward_workspace_bytes(8192, 256000, 2304)
     assert ws > 0 and ws % 8 == 0 and ws <= 16 * 2**20
