@@ -1007,6 +1007,9 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
             constexpr int kLast = kFMaxChunks - 1;
             const int ci = g * 4 + cj;
             if (ci <= kLast && ci < nchunks) {
+              // an accumulator that was pinned to the AGPRs stays there until this very point: otherwise
+              // the compiler moves all of them to ordinary registers (and on to scratch) before the loop
+              if (ci < 16) asm volatile("" : "+a"(acc[ci <= kLast ? ci : kLast]));
               const f32x16& a = acc[ci <= kLast ? ci : kLast];
 #pragma unroll
               for (int r4 = 0; r4 < 4; ++r4) {

@@ -57,13 +57,16 @@ struct Elem<BF16> {
   // The same MFMA with the accumulator pinned to one register file: "a" = the accumulation registers
   // (AGPRs), "v" = the ordinary ones.  For kernels whose accumulators outnumber the 256 AGPRs: the
   // compiler places the results of all MFMA builtins of a function in one file and spills the excess,
-  // so such a kernel writes every one of its MFMAs this way and calls mfma_drain* before other kinds
-  // of instruction read the results.
+  // so such a kernel writes every one of its MFMAs this way.  The compiler cannot see the MFMA inside
+  // the asm statement and inserts none of the wait states the matrix pipeline needs around register
+  // copies it may place next to it, so the statement carries them itself: 5 before (an operand just
+  // written by a move) and 12 after (the result of this 8-pass MFMA read by a move).  They hide under
+  // the 32 cycles the MFMA occupies the pipeline anyway.
   static __device__ __forceinline__ void mfma_agpr(vec8 a, vec8 b, f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 4\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 11" : "+a"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void mfma_vgpr(vec8 a, vec8 b, f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 4\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 11" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
     bf16x2_t v;
@@ -94,10 +97,10 @@ struct Elem<F16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ void mfma_agpr(vec8 a, vec8 b, f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 4\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 11" : "+a"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void mfma_vgpr(vec8 a, vec8 b, f32x16& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("s_nop 4\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 11" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void atomic_add_pair(uint16_t* addr, float lo, float hi) {
     f16x2_t v;
