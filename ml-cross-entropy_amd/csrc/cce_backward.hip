@@ -840,7 +840,15 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       if (tid == 0) sMisc[1] = 0;
       __syncthreads();
       const int* other_ids = IS_DE ? sCellCid : meta.row;
-      const int entry = li + wave;
+      // Waves and entries: with 3 or 4 entries in the trip wave w recomputes entry w over all of D; with
+      // 2 (1) entries, two (four) waves share an entry, each over a half (quarter) of every stage, and the
+      // first of them -- the entry's owner -- sums the partial logits and goes on alone.
+      const int nent = min(4, list_n - li);
+      const int kparts = (nent == 1) ? 4 : ((nent == 2) ? 2 : 1);
+      const int ew = wave / kparts;
+      const int kpart = wave - ew * kparts;
+      const bool owner = (kpart == 0);
+      const int entry = li + ew;
       const bool have_entry = entry < list_n;
       const int entry_id = have_entry ? (use_list ? sList[entry] : (IS_DE ? seg * 4 + entry : seg + entry)) : -1;
 
@@ -855,7 +863,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       // 2 e and 2 e + 1 of a wave belong to entry e), so a short trip moves proportionally less data.
       // A short trip has small stages, so more of them fit the ring and more loads are in flight: a
       // stage holds the rows of the present entries followed by the own rows.
-      const int nent = min(4, list_n - li);
       const int own_off = 32 * nent * kFRowBytes;
       const int slot_bytes = own_off + kFOwnBytes;
       const int ring = (nent >= 3) ? 3 : ((nent == 2) ? 5 : 7);  // slots of this size in the 120 KB ring
@@ -888,9 +895,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         const unsigned char* so = smem + slot * slot_bytes;
         const unsigned char* sw = so + own_off;
         slot = (slot + 1 == ring) ? 0 : slot + 1;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          const auto fo = fstage_frag<T>(so, wave * 32 + l32, kk * 2 + half);
+        const int nkk = 8 / kparts;
+#pragma unroll 2
+        for (int j = 0; j < nkk; ++j) {
+          const int kk = kpart * nkk + j;
+          const auto fo = fstage_frag<T>(so, ew * 32 + l32, kk * 2 + half);
           const auto fw = fstage_frag<T>(sw, l32, kk * 2 + half);
           if (IS_DE) Elem<T>::mfma_vgpr(fo, fw, s);
           else Elem<T>::mfma_vgpr(fw, fo, s);
@@ -899,12 +908,27 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       mfma_drain(s);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the unused prefetches
       __syncthreads();
+      if (kparts > 1) {  // partial logits -> the owner, through the idle ring, in a fixed order
+        float* sRed = reinterpret_cast<float*>(smem);
+        if (!owner) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sRed[(wave * 16 + r) * 64 + lane] = s[r];
+        }
+        __syncthreads();
+        if (owner) {
+          for (int q = 1; q < kparts; ++q) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] += sRed[((wave + q) * 16 + r) * 64 + lane];
+          }
+        }
+        __syncthreads();  // before the product phase refills the ring
+      }
       const int last_chunk_col = d_begin + (nchunks - 1) * kFCols;
 
-      // ---- dz of this wave's 32 x 32 block (lane = token row, registers = classes) ----------------------------
-      {
-        const int mrow = IS_DE ? l32 : wave * 32 + l32;
-        const int* cid32 = IS_DE ? sCellCid + wave * 32 : sOwnCid;
+      // ---- dz of the owner's 32 x 32 block (lane = token row, registers = classes) ----------------------------
+      if (owner) {
+        const int mrow = IS_DE ? l32 : ew * 32 + l32;
+        const int* cid32 = IS_DE ? sCellCid + ew * 32 : sOwnCid;
         const bool big = block_epilogue<T>(p, s, cid32, half, meta.lse2[mrow], meta.g[mrow], meta.h[mrow], meta.tgt[mrow]);
         bool use = have_entry;
         if (IS_DE) {
@@ -918,14 +942,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
           if (IS_DE) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-              const int k = wave * 32 + 8 * r4 + 4 * half;
+              const int k = ew * 32 + 8 * r4 + 4 * half;
               uint2 pk;
               pk.x = Elem<T>::pack2(s[r4 * 4 + 0], s[r4 * 4 + 1]);
               pk.y = Elem<T>::pack2(s[r4 * 4 + 2], s[r4 * 4 + 3]);
               *reinterpret_cast<uint2*>(sDz + l32 * 256 + ((((k >> 3) ^ (l32 & 7)) << 4) | ((k & 7) << 1))) = pk;
             }
           } else {
-            const int k = wave * 32 + l32;
+            const int k = ew * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               const int cls = 8 * (r >> 2) + 4 * half + (r & 3);
@@ -935,11 +959,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
                 float colsum = s[r];
 #pragma unroll
                 for (int off = 16; off >= 1; off >>= 1) colsum += __shfl_xor(colsum, off, 64);
-                if (l32 == 0) sDb[wave * 32 + cls] += colsum;
+                if (l32 == 0) sDb[ew * 32 + cls] += colsum;
               }
             }
           }
-          if (lane == 0) atomicOr(&sMisc[1], 1 << wave);
+          if (lane == 0) atomicOr(&sMisc[1], 1 << ew);
         }
       }
       __syncthreads();
