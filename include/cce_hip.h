@@ -143,15 +143,18 @@ int cce_backward(const void* e, const void* c, const void* bias,
  *
  *   c, bias    the chunk's rows: v classes starting at the caller's offset
  *   lse        [b] float, the LSE over the WHOLE vocabulary
- *   dz         [b, ldz] in `dtype`, row i = valid row i (rows compacted through valids), ldz >= v
+ *   dz         [b, ldz] in `dtype`, or float when dz_is_fp32 (for callers that pass fp32 matrices split
+ *              into 16-bit parts along d and want the gradient at that accuracy); row i = valid row i
+ *              (rows compacted through valids), ldz >= v
  *   target_offset  first class of the chunk (plus the shard start, if any)
- * Needs 16-byte aligned e, c, dz, unit stride_cd, row strides and ldz that are multiples of 8 and d a
+ * Needs 16-byte aligned e, c, dz, unit stride_cd, row strides that are multiples of 8, ldz a multiple of 8
+ * (4 when dz_is_fp32) and d a
  * multiple of 64; anything else returns CCE_ERR_MISALIGNED and the caller uses cce_backward.
  */
 int cce_backward_dz(const void* e, const void* c, const void* bias,
                     const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
                     const int32_t* valids, const int64_t* targets,
-                    void* dz, int64_t ldz,
+                    void* dz, int64_t ldz, int dz_is_fp32,
                     int64_t n_rows, int64_t b, int64_t v, int64_t d,
                     int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
                     float grad_scale, int64_t shift, int64_t target_offset,

@@ -18,7 +18,7 @@ struct DzParams {
   const float* d_out;
   const float* d_lse;
   const int64_t* targets;
-  uint16_t* dz;
+  void* dz;
   int64_t ldz;
   int64_t n_rows, b, v, d;
   int64_t stride_e, stride_cv;
@@ -32,10 +32,12 @@ struct DzParams {
 constexpr int kDzWV = 4, kDzWT = 2, kDzNWV = 2, kDzNWT = 4;  // the forward kernel's wave tiling
 constexpr int kDzThreads = 64 * kDzNWV * kDzNWT;
 constexpr int kDzTile = 256;
-constexpr int kDzStagePitch = 128 * 2 + 16;  // one row of a wave's 32 x 128 block, padded against bank conflicts
+constexpr int kDzStagePitch = 128 * 2 + 16;  // one row of a wave's staged block (128 x 16-bit or 64 x fp32), padded
 constexpr int kDzStageBytes = 32 * kDzStagePitch;
 
-template <typename T, bool GENERAL>
+// OUT32: dz leaves as fp32 (for inputs that are fp32 values split into 16-bit parts along D, whose
+// gradients are wanted at fp32 accuracy): a staged block is then 32 rows x 64 classes.
+template <typename T, bool GENERAL, bool OUT32>
 __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
   using Fast = DmaLogitTile<T, kDzWV, kDzWT, kDzNWV, kDzNWT>;
   static_assert(kDzStageBytes * kDzNWV * kDzNWT <= Fast::LDS_BYTES, "the staging blocks reuse the idle ring");
@@ -125,65 +127,83 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
     for (int ti = 0; ti < kDzWT; ++ti) {
       const float lse2 = r_lse2[ti], g = r_g[ti], gh = r_g[ti] + r_h[ti];
       const int tgt = r_tgt[ti];
+      constexpr int kHalves = OUT32 ? 2 : 1;        // staged blocks per column block
+      constexpr int kViPer = kDzWV / kHalves;       // 32-class blocks per staged block
+      constexpr int kEs = OUT32 ? 4 : 2;            // bytes per stored element
+      constexpr int kPieceElems = 16 / kEs;         // elements per 16-byte piece
 #pragma unroll
-      for (int vi = 0; vi < kDzWV; ++vi) {
+      for (int vh = 0; vh < kHalves; ++vh) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          float dzv[4];
+        for (int vj = 0; vj < kViPer; ++vj) {
+          const int vi = vh * kViPer + vj;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int cl = vi * 32 + 8 * r4 + 4 * half + i;
-            float x = acc[vi][ti][r4 * 4 + i];
-            bool dead = false;
-            if (GENERAL) {
-              const float add = wave_addend[cl];
-              dead = (add == -INFINITY);
-              x = dead ? 0.0f : x + add;
+          for (int r4 = 0; r4 < 4; ++r4) {
+            float dzv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int cl = vi * 32 + 8 * r4 + 4 * half + i;
+              float x = acc[vi][ti][r4 * 4 + i];
+              bool dead = false;
+              if (GENERAL) {
+                const float add = wave_addend[cl];
+                dead = (add == -INFINITY);
+                x = dead ? 0.0f : x + add;
+              }
+              float s2, damp = 1.0f;
+              if (p.sc.on) {
+                const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
+                const float w = __builtin_amdgcn_rcpf(1.0f + t);
+                const float th = 1.0f - 2.0f * w;
+                s2 = p.sc.out_scale * th;
+                damp = 1.0f - th * th;
+              } else {
+                s2 = x * kLog2e;
+              }
+              const float pr = __builtin_amdgcn_exp2f(s2 - lse2);
+              float dz = pr * gh - ((cls0 + cl == tgt) ? g : 0.0f);
+              dz *= damp;
+              dzv[i] = dead ? 0.0f : dz;
             }
-            float s2, damp = 1.0f;
-            if (p.sc.on) {
-              const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
-              const float w = __builtin_amdgcn_rcpf(1.0f + t);
-              const float th = 1.0f - 2.0f * w;
-              s2 = p.sc.out_scale * th;
-              damp = 1.0f - th * th;
+            unsigned char* dst = stage + l32 * kDzStagePitch + (vj * 32 + 8 * r4 + 4 * half) * kEs;
+            if (OUT32) {
+              *reinterpret_cast<float4*>(dst) = make_float4(dzv[0], dzv[1], dzv[2], dzv[3]);
             } else {
-              s2 = x * kLog2e;
+              uint2 pk;
+              pk.x = Elem<T>::pack2(dzv[0], dzv[1]);
+              pk.y = Elem<T>::pack2(dzv[2], dzv[3]);
+              *reinterpret_cast<uint2*>(dst) = pk;
             }
-            const float pr = __builtin_amdgcn_exp2f(s2 - lse2);
-            float dz = pr * gh - ((cls0 + cl == tgt) ? g : 0.0f);
-            dz *= damp;
-            dzv[i] = dead ? 0.0f : dz;
-          }
-          uint2 pk;
-          pk.x = Elem<T>::pack2(dzv[0], dzv[1]);
-          pk.y = Elem<T>::pack2(dzv[2], dzv[3]);
-          *reinterpret_cast<uint2*>(stage + l32 * kDzStagePitch + (vi * 32 + 8 * r4 + 4 * half) * 2) = pk;
-        }
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is private to this wave: no barrier
-      // 32 rows x 256 bytes leave as 16-byte pieces: one instruction covers 4 rows of 256 contiguous bytes
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int j = lane + 64 * k;
-        const int row = j >> 4;
-        const int pc = j & 15;
-        const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kDzStagePitch + pc * 16);
-        const int64_t gi = t0 + wt * (32 * kDzWT) + ti * 32 + row;
-        const int64_t gcol = static_cast<int64_t>(cls0) + pc * 8;
-        if (gi < p.b) {
-          uint16_t* dst = p.dz + gi * p.ldz + gcol;
-          if (!GENERAL || gcol + 8 <= p.v) {
-            *reinterpret_cast<uint4*>(dst) = val;
-          } else {
-            const uint32_t w[4] = {val.x, val.y, val.z, val.w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-              if (gcol + i < p.v) dst[i] = static_cast<uint16_t>(w[i >> 1] >> ((i & 1) * 16));
           }
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is private to this wave: no barrier
+        // 32 rows x 256 bytes leave as 16-byte pieces: one instruction covers 4 rows of 256 contiguous bytes
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const int j = lane + 64 * k;
+          const int row = j >> 4;
+          const int pc = j & 15;
+          const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kDzStagePitch + pc * 16);
+          const int64_t gi = t0 + wt * (32 * kDzWT) + ti * 32 + row;
+          const int64_t gcol = static_cast<int64_t>(cls0) + vh * (32 * kViPer) + pc * kPieceElems;
+          if (gi < p.b) {
+            unsigned char* dst = static_cast<unsigned char*>(p.dz) + (gi * p.ldz + gcol) * kEs;
+            if (!GENERAL || gcol + kPieceElems <= p.v) {
+              *reinterpret_cast<uint4*>(dst) = val;
+            } else if (OUT32) {
+              const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (gcol + i < p.v) reinterpret_cast<uint32_t*>(dst)[i] = w[i];
+            } else {
+              const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (gcol + i < p.v) reinterpret_cast<uint16_t*>(dst)[i] = static_cast<uint16_t>(w[i >> 1] >> ((i & 1) * 16));
+            }
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block is staged
       }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next block is staged
     }
   }
 }
@@ -195,7 +215,7 @@ using namespace cce;
 extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
                                const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
                                const int32_t* valids, const int64_t* targets,
-                               void* dz, int64_t ldz,
+                               void* dz, int64_t ldz, int dz_is_fp32,
                                int64_t n_rows, int64_t b, int64_t v, int64_t d,
                                int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
                                float grad_scale, int64_t shift, int64_t target_offset,
@@ -210,7 +230,7 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
   if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
   // direct-to-LDS main loop and 16-byte stores only
   if (!aligned16(e) || !aligned16(c) || !aligned16(dz) || d % kDmaBK != 0 || stride_e % 8 != 0 ||
-      stride_cv % 8 != 0 || stride_cd != 1 || ldz % 8 != 0)
+      stride_cv % 8 != 0 || stride_cd != 1 || ldz % (dz_is_fp32 ? 4 : 8) != 0)
     return CCE_ERR_MISALIGNED;
 
   DzParams p;
@@ -222,7 +242,7 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
   p.d_out = d_out;
   p.d_lse = d_lse;
   p.targets = targets;
-  p.dz = static_cast<uint16_t*>(dz);
+  p.dz = dz;
   p.ldz = ldz;
   p.n_rows = n_rows;
   p.b = b;
@@ -246,13 +266,17 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
   const bool general = (bias != nullptr) || (v % kDzTile != 0);
   const int grid = p.items_per_xcd * 8;
   hipError_t err;
-#define CCE_LAUNCH_DZ(TT, GE)                                                                     \
+#define CCE_LAUNCH_DZ2(TT, GE, O32)                                                               \
   do {                                                                                            \
-    auto kern = dense_dz_kernel<TT, GE>;                                                          \
+    auto kern = dense_dz_kernel<TT, GE, O32>;                                                     \
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
     if (err != hipSuccess) return status_from_hip(err);                                           \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kDzThreads), lds, stream, p);                       \
+  } while (0)
+#define CCE_LAUNCH_DZ(TT, GE)                                                                     \
+  do {                                                                                            \
+    if (dz_is_fp32) CCE_LAUNCH_DZ2(TT, GE, true); else CCE_LAUNCH_DZ2(TT, GE, false);             \
   } while (0)
   if (dtype == CCE_DTYPE_BF16) {
     if (general) CCE_LAUNCH_DZ(BF16, true); else CCE_LAUNCH_DZ(BF16, false);
@@ -260,5 +284,6 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
     if (general) CCE_LAUNCH_DZ(F16, true); else CCE_LAUNCH_DZ(F16, false);
   }
 #undef CCE_LAUNCH_DZ
+#undef CCE_LAUNCH_DZ2
   return status_from_hip(hipGetLastError());
 }

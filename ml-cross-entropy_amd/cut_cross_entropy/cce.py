@@ -12,6 +12,7 @@ from typing import Optional, Tuple, Union
 import torch
 import torch.amp
 
+from cut_cross_entropy import _hip, fp32_path
 from cut_cross_entropy.cce_backward import cce_backward_kernel
 from cut_cross_entropy.cce_lse_forward import lse_forward
 from cut_cross_entropy.constants import IGNORE_INDEX
@@ -74,22 +75,33 @@ class LinearCrossEntropyFunction(torch.autograd.Function):
             if bias is not None:
                 bias = bias.to(dtype=low)
 
-        lse, _, tile_max = lse_forward(
-            e, c, bias, params.valids, params.softcap, want_tile_max=want_tile_max
-        )
-
         vp = params.vocab_parallel_options
-        neg_dot = indexed_neg_dot_forward_kernel(
-            e=e,
-            c=c,
-            inds=params.targets,
-            bias=bias,
-            shift=params.shift,
-            valids=params.valids,
-            softcap=params.softcap,
-            out_dtype=lse.dtype,
-            target_offset=vp.start if vp is not None else 0,
-        )
+        ctx.fp32 = e.dtype == torch.float32
+        if ctx.fp32:
+            # fp32 values as three bf16 parts along a six times longer reduction axis: fp32_path.py
+            assert c.dtype == torch.float32, "e and c must have the same dtype"
+            _hip.require_gpu_tensor("e", e)
+            e = e.contiguous()
+            lse = fp32_path.fp32_lse(e, c, bias, params.valids, params.softcap)
+            tile_max = None
+            neg_dot = fp32_path.fp32_indexed_neg_dot(
+                e, c, bias, params.targets, params.valids, params.shift, params.softcap,
+                vp.start if vp is not None else 0)
+        else:
+            lse, _, tile_max = lse_forward(
+                e, c, bias, params.valids, params.softcap, want_tile_max=want_tile_max
+            )
+            neg_dot = indexed_neg_dot_forward_kernel(
+                e=e,
+                c=c,
+                inds=params.targets,
+                bias=bias,
+                shift=params.shift,
+                valids=params.valids,
+                softcap=params.softcap,
+                out_dtype=lse.dtype,
+                target_offset=vp.start if vp is not None else 0,
+            )
         nll = neg_dot.add_(lse)
 
         ctx.save_for_backward(e, c, bias, lse, params.targets, params.valids, tile_max)
@@ -134,6 +146,15 @@ class LinearCrossEntropyFunction(torch.autograd.Function):
             grad_lse_out = grad_lse_out.reshape(-1)
 
         vp = params.vocab_parallel_options
+        if ctx.fp32:
+            de, dc, dbias = fp32_path.fp32_backward(
+                e, c, bias, lse, grad_out, grad_lse_out, valids, targets, params.shift,
+                vp.start if vp is not None else 0, params.softcap, grad_scale,
+                ctx.e_info.requires_grad, ctx.c_info.requires_grad,
+                ctx.bias_info is not None and ctx.bias_info.requires_grad)
+            if dbias is not None:
+                dbias = dbias.to(ctx.bias_info.dtype)
+            return de, dc, dbias, None
         de, dc, dbias = cce_backward_kernel(
             do=grad_out,
             dlse=grad_lse_out,

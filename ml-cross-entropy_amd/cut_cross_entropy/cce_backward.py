@@ -81,7 +81,7 @@ def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, 
                 (bias.data_ptr() + v0 * bias.element_size()) if bias is not None else None,
                 lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
                 _hip.ptr(valids), targets.data_ptr(),
-                dz.data_ptr(), ldz,
+                dz.data_ptr(), ldz, 0,
                 e.size(0), B, n, D,
                 e.stride(0), c.stride(0), c.stride(1),
                 float(grad_scale), int(shift), int(target_offset) + v0,

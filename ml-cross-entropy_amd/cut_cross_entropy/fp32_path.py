@@ -1,0 +1,159 @@
+"""fp32 inputs on matrix cores that multiply 16-bit numbers.
+
+gfx950 has no fast fp32 matrix path (the reference leans on Triton's tf32x3 / ieee dot for fp32
+inputs, cce_lse_forward.py:81, constants via tl_utils).  An fp32 value is therefore split into three
+bfloat16 parts, x = hi + mid + lo (8 + 8 + 8 significant bits), and the product of two such sums is
+taken as the six leading terms
+
+    hi*hi + hi*mid + mid*hi + mid*mid + hi*lo + lo*hi          (what is left is below 2^-24 relative)
+
+which is ONE 16-bit contraction over a six times longer reduction axis: E' = [hi hi mid mid hi lo] and
+C' = [hi mid hi mid lo hi] side by side along D.  The unchanged bf16 kernels then produce logits of fp32
+accuracy (their accumulators are fp32).  A bias rides along as three more columns (ones in E', the
+three parts of the bias in C').  The vocabulary is walked in chunks so that the widened copy of the
+classifier stays small; chunk log-sum-exps are merged with logaddexp.
+
+Backward: the gradient filter threshold of fp32 is far below anything a soft-max produces, so the
+backward is the unfiltered one: the dz kernel runs on the widened matrices and writes dz as fp32, and
+the two products are fp32 GEMMs on the original matrices.
+"""
+
+from typing import Optional, Tuple
+
+import torch
+
+from cut_cross_entropy import _hip
+from cut_cross_entropy.cce_lse_forward import lse_forward
+
+_WIDE_C_BYTES = 1 << 29   # widened classifier chunk
+_DZ_ELEMS = 1 << 25       # fp32 dz chunk (128 MB)
+
+
+def split3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    hi = x.to(torch.bfloat16)
+    r = x - hi.to(torch.float32)
+    mid = r.to(torch.bfloat16)
+    lo = (r - mid.to(torch.float32)).to(torch.bfloat16)
+    return hi, mid, lo
+
+
+def _padded_width(d: int, has_bias: bool) -> int:
+    w = 6 * d + (3 if has_bias else 0)
+    return (w + 63) // 64 * 64
+
+
+def widen_e(e: torch.Tensor, has_bias: bool) -> torch.Tensor:
+    """[N, D] fp32 -> [N, Dp] bf16 = [hi hi mid mid hi lo (1 1 1) 0 ...]."""
+    n, d = e.shape
+    hi, mid, lo = split3(e)
+    out = torch.zeros((n, _padded_width(d, has_bias)), dtype=torch.bfloat16, device=e.device)
+    for k, part in enumerate((hi, hi, mid, mid, hi, lo)):
+        out[:, k * d : (k + 1) * d] = part
+    if has_bias:
+        out[:, 6 * d : 6 * d + 3] = 1.0
+    return out
+
+
+def widen_c(c: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """[V, D] fp32 (+ [V] bias) -> [V, Dp] bf16 = [hi mid hi mid lo hi (b_hi b_mid b_lo) 0 ...]."""
+    v, d = c.shape
+    hi, mid, lo = split3(c)
+    out = torch.zeros((v, _padded_width(d, bias is not None)), dtype=torch.bfloat16, device=c.device)
+    for k, part in enumerate((hi, mid, hi, mid, lo, hi)):
+        out[:, k * d : (k + 1) * d] = part
+    if bias is not None:
+        for k, part in enumerate(split3(bias.to(torch.float32))):
+            out[:, 6 * d + k] = part
+    return out
+
+
+def _chunk(v: int, per_class_bytes: int, budget: int) -> int:
+    return max(256, min(v, (budget // max(per_class_bytes, 1)) // 256 * 256))
+
+
+def fp32_lse(e, c, bias, valids, softcap) -> torch.Tensor:
+    """Log-sum-exp of the valid rows over the whole vocabulary, fp32 accurate."""
+    e6 = widen_e(e, bias is not None)
+    n_valid = valids.numel() if valids is not None else e.size(0)
+    lse = torch.full((n_valid,), float("-inf"), dtype=torch.float32, device=e.device)
+    vc = _chunk(c.size(0), e6.size(1) * 2, _WIDE_C_BYTES)
+    for v0 in range(0, c.size(0), vc):
+        c6 = widen_c(c[v0 : v0 + vc], bias[v0 : v0 + vc] if bias is not None else None)
+        part, _, _ = lse_forward(e6, c6, None, valids, softcap)
+        lse = torch.logaddexp(lse, part)
+    return lse
+
+
+def fp32_indexed_neg_dot(e, c, bias, targets, valids, shift, softcap, target_offset) -> torch.Tensor:
+    """-(soft-capped logit of the target) per valid row, 0 where the target is not a class of this
+    shard (the semantics of the indexed-dot kernel).  O(rows x D) work: plain fp32 arithmetic."""
+    n = e.size(0)
+    rows = valids.to(torch.int64) if valids is not None else torch.arange(n, device=e.device)
+    tpos = rows + int(shift)
+    ok = tpos < n
+    t = torch.where(ok, targets[tpos.clamp_max(n - 1)] - int(target_offset), torch.full_like(tpos, -1))
+    ok = ok & (t >= 0) & (t < c.size(0))
+    tc = t.clamp(0, c.size(0) - 1)
+    logit = (e[rows] * c[tc]).sum(dim=1)
+    if bias is not None:
+        logit = logit + bias[tc].to(torch.float32)
+    if softcap is not None:
+        logit = torch.tanh(logit / softcap) * softcap
+    return torch.where(ok, -logit, torch.zeros_like(logit))
+
+
+def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offset, softcap, grad_scale,
+                  want_de, want_dc, want_dbias):
+    """(dE, dC, dBias) in fp32: dz of a vocabulary chunk from the HIP kernel (fp32 output), products as
+    fp32 GEMMs."""
+    lib = _hip.load()
+    dev = e.device
+    n, d = e.shape
+    v = c.size(0)
+    rows = valids.to(torch.int64) if valids is not None else None
+    n_valid = rows.numel() if rows is not None else n
+    de = torch.zeros_like(e) if want_de else None
+    dc = torch.zeros_like(c) if want_dc else None
+    dbias = torch.zeros((v,), dtype=torch.float32, device=dev) if want_dbias else None
+    if n_valid == 0 or not (want_de or want_dc or want_dbias):
+        return de, dc, dbias
+    e6 = widen_e(e, bias is not None)
+    e_rows = e if rows is None else e.index_select(0, rows)
+    de_acc = torch.zeros((n_valid, d), dtype=torch.float32, device=dev) if want_de else None
+    vc = min(_chunk(v, e6.size(1) * 2, _WIDE_C_BYTES), _chunk(v, n_valid * 4, _DZ_ELEMS * 4))
+    dz_buf = torch.empty((n_valid * ((min(vc, v) + 3) // 4 * 4),), dtype=torch.float32, device=dev)
+    do = do.to(torch.float32).contiguous().view(-1)
+    dlse = dlse.to(torch.float32).contiguous().view(-1) if dlse is not None else None
+    targets = targets.to(torch.int64).contiguous()
+    stream = _hip.current_stream_ptr(dev)
+    for v0 in range(0, v, vc):
+        m = min(vc, v - v0)
+        ldz = (m + 3) // 4 * 4
+        dz = dz_buf[: n_valid * ldz].view(n_valid, ldz)
+        c_chunk = c[v0 : v0 + m]
+        c6 = widen_c(c_chunk, bias[v0 : v0 + m] if bias is not None else None)
+        with torch.cuda.device(dev):
+            status = lib.cce_backward_dz(
+                e6.data_ptr(), c6.data_ptr(), None,
+                lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
+                _hip.ptr(valids), targets.data_ptr(),
+                dz.data_ptr(), ldz, 1,
+                n, n_valid, m, e6.size(1),
+                e6.stride(0), c6.stride(0), c6.stride(1),
+                float(grad_scale), int(shift), int(target_offset) + v0,
+                float(softcap) if softcap is not None else 0.0, _hip.DTYPE_CODES[torch.bfloat16], stream,
+            )
+        _hip.check(status, "cce_backward_dz")
+        dzv = dz[:, :m]
+        if de_acc is not None:
+            de_acc.addmm_(dzv, c_chunk)
+        if dc is not None:
+            torch.mm(dzv.t(), e_rows, out=dc[v0 : v0 + m])
+        if dbias is not None:
+            dbias[v0 : v0 + m] = dzv.sum(dim=0)
+    if de is not None:
+        if rows is None:
+            de.copy_(de_acc)
+        else:
+            de.index_copy_(0, rows, de_acc)
+    return de, dc, dbias

@@ -202,7 +202,7 @@ def test_backward_dz_abi(dtype, softcap, has_bias, with_dlse, shape):
         dz = torch.full((B + 3, ldz), 7.0, dtype=dtype, device=dev)
         st = lib.cce_backward_dz(
             p(ed), cd[v0:v1].data_ptr(), (bd.data_ptr() + 2 * v0) if bd is not None else None,
-            p(lsed), p(dod), 0, p(dld), p(vd), p(td), p(dz), ldz,
+            p(lsed), p(dod), 0, p(dld), p(vd), p(td), p(dz), ldz, 0,
             N, B, n, D, ed.stride(0), cd.stride(0), cd.stride(1),
             0.5, 0, v0, softcap or 0.0, 0 if dtype == torch.bfloat16 else 1,
             torch.cuda.current_stream().cuda_stream)
@@ -230,6 +230,6 @@ def test_backward_dz_rejects_layouts_it_cannot_stream():
     t = torch.zeros((64,), dtype=torch.int64, device=dev)
     dz = torch.zeros((64, 128), dtype=torch.bfloat16, device=dev)
     st = lib.cce_backward_dz(e.data_ptr(), c.data_ptr(), None, lse.data_ptr(), lse.data_ptr(), 0, None, None,
-                             t.data_ptr(), dz.data_ptr(), 128, 64, 64, 128, 72, 72, 72, 1, 1.0, 0, 0, 0.0, 0,
+                             t.data_ptr(), dz.data_ptr(), 128, 0, 64, 64, 128, 72, 72, 72, 1, 1.0, 0, 0, 0.0, 0,
                              torch.cuda.current_stream().cuda_stream)
     assert st == 10004  # CCE_ERR_MISALIGNED

@@ -240,3 +240,71 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     ed2, cd2 = e2.cuda().requires_grad_(True), c2.cuda().requires_grad_(True)
     linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
     assert len(calls) == 1
+
+
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("shift", [0, 1])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (252, 507, 123), (1024, 4096, 256)])
+def test_fp32_inputs_match_fp64_oracle(softcap, has_bias, shift, shape):
+    """fp32 inputs (three bf16 parts along a widened reduction axis, fp32 dz, fp32 GEMMs): the
+    reference's tolerances for this dtype -- 1e-5 on the loss (tests/test_cce_loss_forward.py:47),
+    5e-4 on the gradients (tests/test_cce_loss_backward.py:82) -- against the fp64 dense oracle, with the
+    fp32 dense result as the yardstick of the reference's criterion."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, torch.float32, seed=9, bias=has_bias, invalid_frac=0.2)
+    if bias is not None:
+        bias = bias * 10  # make the bias matter
+
+    def dense(dtype):
+        el = e.detach().clone().to(dtype).requires_grad_(True)
+        cl = c.detach().clone().to(dtype).requires_grad_(True)
+        bl = bias.detach().clone().to(dtype).requires_grad_(True) if bias is not None else None
+        loss, _ = dense_lce.dense_linear_cross_entropy(el, cl, t, bias=bl, softcap=softcap, shift=shift,
+                                                       reduction="none")
+        (loss * w.to(dtype)[..., shift:]).sum().backward()
+        return loss.detach(), el.grad, cl.grad, (bl.grad if bl is not None else None)
+
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn((N,), generator=g)
+    gt = dense(torch.float64)
+    ref = dense(torch.float32)
+
+    ed = e.cuda().requires_grad_(True)
+    cd = c.cuda().requires_grad_(True)
+    bd = bias.cuda().requires_grad_(True) if bias is not None else None
+    loss = linear_cross_entropy(ed, cd, t.cuda(), bias=bd, softcap=softcap, shift=shift, reduction="none")
+    assert loss.dtype == torch.float32 and ed.dtype == torch.float32
+    (loss * w.cuda()[..., shift:]).sum().backward()
+    assert_no_worse(gt[0], ref[0], loss.detach(), 1e-5, "loss")
+    assert_no_worse(gt[1], ref[1], ed.grad, 5e-4, "dE")
+    assert_no_worse(gt[2], ref[2], cd.grad, 5e-4, "dC")
+    if bias is not None:
+        assert_no_worse(gt[3], ref[3], bd.grad, 5e-4, "dBias")
+    ignored = t == IGNORE_INDEX
+    if shift:
+        ignored = torch.cat([ignored[shift:], torch.ones(shift, dtype=torch.bool)])
+    assert (ed.grad.cpu()[ignored] == 0).all()
+
+
+def test_fp32_mean_and_lse_and_shard():
+    from cut_cross_entropy import VocabParallelOptions, linear_cross_entropy
+    from oracle import dense_lce
+
+    e, c, t, _ = make_inputs(300, 1000, 64, torch.float32, seed=12)
+    want, want_lse = dense_lce.dense_linear_cross_entropy(e.double(), c.double(), t, return_lse=True)
+    got, got_lse = linear_cross_entropy(e.cuda(), c.cuda(), t.cuda(), return_lse=True)
+    assert abs(got.item() - want.item()) <= 1e-5
+    assert torch.allclose(got_lse.cpu().double(), want_lse, atol=1e-5, rtol=0)
+    # a vocabulary shard: shard-local loss = lse over the shard - target logit (0 for foreign targets)
+    s0, s1 = 200, 712
+    one = linear_cross_entropy(e.cuda(), c[s0:s1].cuda(), t.cuda(), reduction="none",
+                               vocab_parallel_options=VocabParallelOptions(s0, s1))
+    logits = e.double() @ c[s0:s1].double().T
+    inside = (t >= s0) & (t < s1)
+    corr = torch.where(inside, logits.gather(1, (t - s0).clamp(0, s1 - s0 - 1).view(-1, 1)).squeeze(1),
+                       torch.zeros(300, dtype=torch.float64))
+    assert torch.allclose(one.cpu().double(), torch.logsumexp(logits, 1) - corr, atol=2e-5, rtol=0)
