@@ -351,3 +351,36 @@ def test_strided_classifier_and_lse_kernel_logit_avg():
     logits = dense_lce._dense_logits(e.cpu(), c.cpu(), None, 20.0, torch.float64)
     assert torch.allclose(lse.cpu().double(), torch.logsumexp(logits, -1), rtol=1e-4, atol=1e-4)
     assert torch.allclose(la.cpu().double(), logits.mean(0), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("impl", ["cce", "cce_exact"])
+def test_classifier_beyond_two_to_the_31_elements(impl):
+    """A classifier of 2.2e9 elements (4.4 GB of bf16): row offsets into C and dC pass 2^31 both in bytes and in
+    elements.  Half of the labels sit in the classes above element offset 2^31, the inputs are peaked on
+    their labels so that the sparse kernels run under impl="cce".  Checked against dense fp32 torch."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, D, V = 512, 8192, 270336
+    first_high = (2**31) // D
+    assert first_high < V - 1024
+    g = torch.Generator(device=DEV).manual_seed(11)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (N,), generator=g, device=DEV)
+    t[::2] = torch.randint(first_high, V, (N // 2,), generator=g, device=DEV)
+    e = (2.0 * c[t].float() + 0.5 * torch.randn((N, D), generator=g, device=DEV)).to(torch.bfloat16)
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    loss, lse = linear_cross_entropy(ed, cd, t, impl=impl, return_lse=True)
+    loss.backward()
+
+    d_out = torch.full((N,), 1.0 / N, device=DEV)
+    want_lse, de, dc, _ = _oracle_on_gpu(e, c, t, None, d_out, None, None,
+                                         filter_eps=2.0**-12 if impl == "cce" else None)
+    from oracle import dense_lce
+
+    assert torch.allclose(lse, want_lse, rtol=1e-3, atol=1e-3)
+    want_loss = (want_lse + dense_lce.dense_indexed_neg_dot(e, c, t, None, None, torch.float32)).mean()
+    assert abs(loss.item() - want_loss.item()) <= 1e-3 * abs(want_loss.item())
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad[first_high:], dc[first_high:]) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
