@@ -40,6 +40,15 @@ def _mm_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         return torch.mm(a, b).to(torch.float32)
 
 
+def _addmm_fp32(acc: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``acc + a @ b`` in fp32 (acc fp32, a and b 16-bit), the addition inside the GEMM where the build has it."""
+    try:
+        return torch.addmm(acc, a, b, out_dtype=torch.float32, out=acc)
+    except (TypeError, RuntimeError):
+        acc += _mm_fp32(a, b)
+        return acc
+
+
 def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
     """The unfiltered backward runs as (dz kernel + library GEMMs) when nothing that is asked for is
     filtered and the layout suits the direct-to-LDS kernel."""
@@ -90,7 +99,7 @@ def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, 
         _hip.check(status, "cce_backward_dz")
         dzv = dz[:, :n]
         if de_acc is not None:
-            de_acc += _mm_fp32(dzv, c_chunk)
+            de_acc = _addmm_fp32(de_acc, dzv, c_chunk)
         if dc is not None:
             if dc.dtype == torch.float32:
                 dc[v0 : v0 + n] = _mm_fp32(dzv.t(), e_rows)
