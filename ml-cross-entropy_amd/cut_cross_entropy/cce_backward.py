@@ -214,7 +214,17 @@ def cce_backward_kernel(
         # once (dC, dBias) or summed in a separate fp32 buffer (dE): no fp32 gradient buffers are needed
         de_dtype, dc_dtype = e_info.dtype, c_info.dtype
     de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
-    dc = torch.zeros_like(c, dtype=dc_dtype) if c_info.requires_grad else None
+    dc = None
+    if c_info.requires_grad:
+        dc = torch.zeros_like(c, dtype=dc_dtype)
+        if dc.stride() != c.stride():
+            # a view with gaps between its rows or columns (zeros_like packs those): the kernels address C and
+            # dC with one pair of strides, so dC gets the layout of c, or c is packed if its elements overlap
+            (s_small, n_small), (s_large, _) = sorted(zip(c.stride(), c.size()))
+            if s_small >= 1 and s_large >= s_small * n_small:
+                dc = torch.empty_strided(c.size(), c.stride(), dtype=dc_dtype, device=dev).zero_()
+            else:
+                c = c.contiguous()
     dbias = None
     if bias is not None:
         assert bias_info is not None

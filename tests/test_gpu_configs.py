@@ -384,3 +384,38 @@ def test_classifier_beyond_two_to_the_31_elements(impl):
     assert _rel_err(ed.grad, de) <= 1e-2
     assert _rel_err(cd.grad[first_high:], dc[first_high:]) <= 1e-2
     assert _rel_err(cd.grad, dc) <= 1e-2
+
+
+@pytest.mark.parametrize("layout", ["row_gaps", "transposed"])
+@pytest.mark.parametrize("impl", ["cce", "cce_exact"])
+def test_backward_with_a_classifier_that_is_a_view(layout, impl):
+    """c as a column slice of a wider matrix (gaps between rows) and as the transpose of a [D, V] matrix
+    (unit stride along the classes): loss and gradients against the dense oracle, gradient in c's shape."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    N, D, V = 384, 128, 1500
+    e, c, t, _ = _gen(N, D, V, seed=12, c_std=0.1)
+    eo = e.float().requires_grad_(True)
+    co = c.float().requires_grad_(True)
+    want, _ = dense_lce.dense_linear_cross_entropy(eo, co, t, softcap=15.0)
+    want.backward()
+
+    ed = e.to(DEV).requires_grad_(True)
+    if layout == "row_gaps":
+        base = torch.zeros((V, D + 64), dtype=c.dtype, device=DEV)
+        base[:, :D] = c.to(DEV)
+        base.requires_grad_(True)
+        cd = base[:, :D]
+    else:
+        base = c.to(DEV).t().contiguous().requires_grad_(True)  # [D, V]
+        cd = base.t()
+    assert not cd.is_contiguous()
+    loss = linear_cross_entropy(ed, cd, t.to(DEV), softcap=15.0, impl=impl, filter_eps=None if impl == "cce_exact" else 0.0)
+    loss.backward()
+    assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+    got_dc = base.grad[:, :D] if layout == "row_gaps" else base.grad.t()
+    assert _rel_err(ed.grad.cpu(), eo.grad) <= 1e-2
+    assert _rel_err(got_dc.cpu(), co.grad) <= 1e-2
+    if layout == "row_gaps":
+        assert (base.grad[:, D:] == 0).all()
