@@ -25,7 +25,7 @@ PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk x 2.4 GHz, dense
 # HBM bytes per launch of lse_forward_kernel at workload c2, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0
 # + WRITE_SIZE x 1.0, factors from a 1 GiB copy in the same runs; summary in profiles/).  A counter cannot be
 # read from inside this script, so the figure of the last profiled build is reported unless --traffic is given.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.523e10}
+MEASURED_TRAFFIC_BYTES = {"c2": 1.446e10}
 
 
 def make_workload(name, device):
