@@ -116,26 +116,8 @@ struct Elem<F16> {
 __device__ __forceinline__ void mfma_drain(f32x16& c) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(c)); }
 __device__ __forceinline__ void mfma_drain_all() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory"); }
 
-// Add `val` to one 16-bit float in global memory through a compare-and-swap on the aligned
-// 32-bit word that contains it (used where a packed two-element atomic would be misaligned).
-template <typename T>
-__device__ __forceinline__ void atomic_add_16(uint16_t* addr, float val) {
-  uintptr_t a = reinterpret_cast<uintptr_t>(addr);
-  unsigned int* word = reinterpret_cast<unsigned int*>(a & ~static_cast<uintptr_t>(3));
-  const bool high = (a & 2) != 0;
-  unsigned int old = *word, assumed;
-  do {
-    assumed = old;
-    uint16_t cur = high ? static_cast<uint16_t>(assumed >> 16) : static_cast<uint16_t>(assumed & 0xffffu);
-    uint16_t upd = Elem<T>::from_float(Elem<T>::to_float(cur) + val);
-    unsigned int next = high ? ((assumed & 0x0000ffffu) | (static_cast<unsigned int>(upd) << 16))
-                             : ((assumed & 0xffff0000u) | upd);
-    old = atomicCAS(word, assumed, next);
-  } while (old != assumed);
-}
-
-// Soft-capping in the log2 domain.  For a raw logit x returns s * log2(e) with
-// s = softcap * tanh(x / softcap) (or s = x when off) and the tanh value itself.
+// Constants of soft-capping in the log2 domain: for a raw logit x the kernels form
+// s * log2(e) = out_scale * tanh(x / softcap) with tanh(u) = 1 - 2 / (1 + exp2(x * in_scale)).
 struct Softcap {
   float in_scale;   // 2 * log2(e) / softcap
   float out_scale;  // softcap * log2(e)
@@ -148,18 +130,6 @@ __host__ __device__ inline Softcap make_softcap(float softcap) {
   s.in_scale = s.on ? 2.0f * kLog2e / softcap : 0.0f;
   s.out_scale = s.on ? softcap * kLog2e : 0.0f;
   return s;
-}
-
-// tanh(y) = 1 - 2 / (1 + exp(2 y)); exp2 overflow gives 1, underflow gives -1.
-__device__ __forceinline__ float softcap_log2(const Softcap& sc, float x, float& th) {
-  if (sc.on) {
-    float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
-    float w = __builtin_amdgcn_rcpf(1.0f + t);
-    th = 1.0f - 2.0f * w;
-    return sc.out_scale * th;
-  }
-  th = 0.0f;
-  return x * kLog2e;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -222,12 +192,6 @@ struct RowLoader {
     }
   }
 };
-
-template <typename T>
-__device__ __forceinline__ typename Elem<T>::vec8 lds_frag(const unsigned char* lds, int row, int chunk) {
-  uint4 v = *reinterpret_cast<const uint4*>(lds + row * kRowBytes + ((chunk ^ (row & 7)) << 4));
-  return __builtin_bit_cast(typename Elem<T>::vec8, v);
-}
 
 // ---------------------------------------------------------------------------------------------
 // One logit tile: acc[vi][ti] += C_tile (TILE_V x D) * E_tile^T (D x TILE_T), both streamed through
@@ -307,188 +271,6 @@ struct LogitTile {
 };
 
 // ---------------------------------------------------------------------------------------------
-// Fast logit tile for the common case (16-byte aligned rows, unit column stride, D % 32 == 0).
-//
-// Differences to LogitTile: 32 reduction columns per LDS stage (64-byte rows, chunk swizzle with
-// (row >> 2) & 3), branch-free loads (a row outside the matrix is clamped to the last valid row:
-// its logits are discarded by the caller), and the global loads for stage k + 2 are issued before
-// the MFMAs of stage k, so two stages of HBM / L2 latency are hidden behind compute.
-// `lds` must hold 2 * (TILE_V + TILE_T) * 64 bytes.
-// ---------------------------------------------------------------------------------------------
-constexpr int kFastBK = 32;
-constexpr int kFastRowBytes = 64;
-
-template <int ROWS, int NT>
-struct FastLoader {
-  static constexpr int NQ = ROWS * 4 / NT;
-  static constexpr int ROWSTEP = NT / 4;
-  static_assert(ROWS * 4 % NT == 0, "tile rows must divide evenly over the threads");
-  static_assert(ROWSTEP % 16 == 0, "swizzle must not depend on q");
-  const uint16_t* ptr[NQ];  // row base + this thread's 8-element chunk; always a readable address
-  struct Regs {
-    uint4 v[NQ];
-  };
-
-  __device__ __forceinline__ Regs load(int k0) const {
-    Regs r;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) r.v[q] = *reinterpret_cast<const uint4*>(ptr[q] + k0);
-    return r;
-  }
-  static __device__ __forceinline__ void store(const Regs& r, unsigned char* lds) {
-    const int row0 = threadIdx.x >> 2;
-    const int chunk = (threadIdx.x & 3) ^ ((row0 >> 2) & 3);
-#pragma unroll
-    for (int q = 0; q < NQ; ++q)
-      *reinterpret_cast<uint4*>(lds + (row0 + q * ROWSTEP) * kFastRowBytes + (chunk << 4)) = r.v[q];
-  }
-};
-
-template <typename T, int WV, int WT, int NWV, int NWT>
-struct FastLogitTile {
-  static constexpr int TILE_V = 32 * WV * NWV;
-  static constexpr int TILE_T = 32 * WT * NWT;
-  static constexpr int NT = 64 * NWV * NWT;
-  static constexpr int STAGE_BYTES = (TILE_V + TILE_T) * kFastRowBytes;
-  static constexpr int LDS_BYTES = 3 * STAGE_BYTES;
-  using CLoader = FastLoader<TILE_V, NT>;
-  using ELoader = FastLoader<TILE_T, NT>;
-  using vec8 = typename Elem<T>::vec8;
-
-  struct Frags {
-    vec8 a[WV];
-    vec8 b[WT];
-  };
-
-  // MFMA operands of one 16-column step: WV class fragments and WT row fragments of this wave.
-  static __device__ __forceinline__ Frags read_frags(const unsigned char* lds, int stage_off, int kk, int coff0,
-                                                     int eoff0, int sw, int half) {
-    Frags f;
-    const int chunk = (((kk * 2 + half) ^ sw) << 4);
-    const unsigned char* cb = lds + stage_off + coff0 + chunk;
-    const unsigned char* eb = lds + stage_off + eoff0 + chunk;
-#pragma unroll
-    for (int vi = 0; vi < WV; ++vi)
-      f.a[vi] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(cb + vi * 32 * kFastRowBytes));
-#pragma unroll
-    for (int ti = 0; ti < WT; ++ti)
-      f.b[ti] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(eb + ti * 32 * kFastRowBytes));
-    return f;
-  }
-
-  static __device__ __forceinline__ void mma(f32x16 (&acc)[WV][WT], const Frags& f) {
-#pragma unroll
-    for (int vi = 0; vi < WV; ++vi)
-#pragma unroll
-      for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
-  }
-
-  // Issue order of one stage: the memory instructions are spread evenly between the MFMAs, so that
-  // the matrix pipe never waits for a burst of loads to issue.  First half: the global loads, then
-  // the fragment reads of step 1; second half: the LDS stores, then the fragment reads of the next
-  // stage (measured: this order beats fragment reads first).
-  template <int OTHER_MASK>
-  static __device__ __forceinline__ void interleave_half() {
-    constexpr int kMfma = 0x008, kDsRead = 0x100;
-    constexpr int nmem = CLoader::NQ + ELoader::NQ;  // global loads = LDS stores per stage
-    constexpr int nfrag = WV + WT;                    // fragment reads per step
-    constexpr int nmma = WV * WT;
-    constexpr int total = nmem + nfrag;
-#pragma unroll
-    for (int i = 0; i < nmma; ++i) {
-      __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-#pragma unroll
-      for (int j = i * total / nmma; j < (i + 1) * total / nmma; ++j) {
-        if (j < nmem) __builtin_amdgcn_sched_group_barrier(OTHER_MASK, 1, 0);
-        else __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
-      }
-    }
-  }
-  static __device__ __forceinline__ void interleave() {
-    interleave_half<0x020>();  // VMEM reads
-    interleave_half<0x200>();  // DS writes
-  }
-
-  // Software pipeline, one barrier per 32-column stage s (LDS ring of three stages, two register
-  // sets for data in flight, two fragment sets):
-  //     issue global loads of stage s + 3          -> register set (s + 1) % 2
-  //     read fragments (s, step 1); MFMAs (s, step 0)
-  //     LDS[(s + 2) % 3] <- register set s % 2      (stage s + 2, issued one and a half trips ago)
-  //     read fragments (s + 1, step 0); MFMAs (s, step 1)
-  //     barrier
-  // Every LDS read is issued a full MFMA group before its use, every global load about two stages
-  // before its LDS store.  Prefetches past the last stage re-read it (never consumed), so the loop
-  // has no branches.
-  static __device__ __forceinline__ void run(f32x16 (&acc)[WV][WT], const CLoader& cl, const ELoader& el,
-                                             unsigned char* lds, int D) {
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int wv = wave / NWT;
-    const int wt = wave % NWT;
-    const int l32 = lane & 31;
-    const int half = lane >> 5;
-    const int sw = (l32 >> 2) & 3;
-    const int coff0 = (wv * WV * 32 + l32) * kFastRowBytes;
-    const int eoff0 = (TILE_V + wt * WT * 32 + l32) * kFastRowBytes;
-
-#pragma unroll
-    for (int vi = 0; vi < WV; ++vi)
-#pragma unroll
-      for (int ti = 0; ti < WT; ++ti)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[vi][ti][r] = 0.0f;
-
-    const int nk = D / kFastBK;
-    const int last = (nk - 1) * kFastBK;
-    typename CLoader::Regs rc0 = cl.load(0);
-    typename ELoader::Regs re0 = el.load(0);
-    typename CLoader::Regs rc1 = cl.load(min(kFastBK, last));
-    typename ELoader::Regs re1 = el.load(min(kFastBK, last));
-    CLoader::store(rc0, lds);
-    ELoader::store(re0, lds + TILE_V * kFastRowBytes);
-    rc0 = cl.load(min(2 * kFastBK, last));
-    re0 = el.load(min(2 * kFastBK, last));
-    CLoader::store(rc1, lds + STAGE_BYTES);
-    ELoader::store(re1, lds + STAGE_BYTES + TILE_V * kFastRowBytes);
-    __syncthreads();
-
-    int o0 = 0, o1 = STAGE_BYTES, o2 = 2 * STAGE_BYTES;  // LDS offsets of stages s, s + 1, s + 2
-    Frags f0 = read_frags(lds, o0, 0, coff0, eoff0, sw, half);
-    Frags f1;
-
-#define CCE_FAST_STAGE(S, RC_NEW, RE_NEW, RC_OLD, RE_OLD)                                        \
-  do {                                                                                            \
-    const int kn = min(((S) + 3) * kFastBK, last);                                                \
-    RC_NEW = cl.load(kn);                                                                         \
-    RE_NEW = el.load(kn);                                                                         \
-    f1 = read_frags(lds, o0, 1, coff0, eoff0, sw, half);                                          \
-    mma(acc, f0);                                                                                 \
-    CLoader::store(RC_OLD, lds + o2);                                                             \
-    ELoader::store(RE_OLD, lds + o2 + TILE_V * kFastRowBytes);                                    \
-    f0 = read_frags(lds, o1, 0, coff0, eoff0, sw, half);                                          \
-    mma(acc, f1);                                                                                 \
-    interleave();                                                                                 \
-    __syncthreads();                                                                              \
-    const int t = o0;                                                                             \
-    o0 = o1;                                                                                      \
-    o1 = o2;                                                                                      \
-    o2 = t;                                                                                       \
-  } while (0)
-
-    const int pairs = nk >> 1;
-#pragma unroll 1
-    for (int pi = 0; pi < pairs; ++pi) {
-      CCE_FAST_STAGE(2 * pi, rc1, re1, rc0, re0);
-      CCE_FAST_STAGE(2 * pi + 1, rc0, re0, rc1, re1);
-    }
-    if (nk & 1) {
-      CCE_FAST_STAGE(nk - 1, rc1, re1, rc0, re0);
-    }
-#undef CCE_FAST_STAGE
-  }
-};
-
-// ---------------------------------------------------------------------------------------------
 // Logit tile with direct global -> LDS loads (gfx950 `global_load_lds_dwordx4`): the data never
 // passes through registers and no wave spends issue slots on LDS stores.
 //
@@ -526,7 +308,6 @@ struct DmaLogitTile {
   static constexpr int NQC = TILE_V / 8 / NW;  // loads per wave and stage that fetch class rows
   static constexpr int NQE = TILE_T / 8 / NW;  // ... token rows
   static constexpr int NQ = NQC + NQE;
-  static constexpr int NSTEP = kDmaBK / 16;
   // The loads of a stage are issued in two groups, one load after every second MFMA: [0, QA) under step 3
   // of the stage before last and [QA, NQ) under step 0 of the last, which leaves them steps 1 and 2 to land
   // (measured: 1 % faster than three groups over steps 3, 0 and 1 with one step to land).
@@ -565,13 +346,6 @@ struct DmaLogitTile {
     for (int ti = 0; ti < WT; ++ti)
       f.b[ti] = __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(eb + ti * 32 * kDmaRowBytes));
     return f;
-  }
-
-  static __device__ __forceinline__ void mma(f32x16 (&acc)[WV][WT], const Frags& f) {
-#pragma unroll
-    for (int vi = 0; vi < WV; ++vi)
-#pragma unroll
-      for (int ti = 0; ti < WT; ++ti) acc[vi][ti] = Elem<T>::mfma(f.a[vi], f.b[ti], acc[vi][ti]);
   }
 
   // Issue load q of one stage (columns [k0, k0 + 64)) into LDS stage `stage_off`.
