@@ -5,11 +5,11 @@ README.md:301-311); arguments are parsed with argparse.
 """
 
 import argparse
+import dataclasses
 import functools
 import gc
+import pathlib
 import time
-from dataclasses import asdict
-from pathlib import Path
 from typing import Optional
 
 import pandas as pd
@@ -21,73 +21,85 @@ from cut_cross_entropy.constants import IGNORE_INDEX
 
 from . import data, memory
 
+# what each kind times: (forward inside the timed region, backward run at all)
+KINDS = {"loss-fw": (True, False), "loss-bw": (False, True), "loss-fw-bw": (True, True)}
+
 
 def baseline(e, c, targets, softcap: Optional[float] = None, ignore_index: int = IGNORE_INDEX, reduction="mean"):
     """Logits in HBM, then the framework's cross-entropy (ref: benchmark/__main__.py:20-34)."""
-    logits = e @ c.T
+    z = e @ c.T
     if softcap is not None:
-        logits = torch.tanh(logits / softcap) * softcap
-    return F.cross_entropy(logits.float(), targets, ignore_index=ignore_index, reduction=reduction)
+        z = softcap * torch.tanh(z / softcap)
+    return F.cross_entropy(z.float(), targets, reduction=reduction, ignore_index=ignore_index)
 
 
-def clear_grad_fn(e, c, *args, **kwargs):
-    e.grad = c.grad = None
+def _drop_grads(e, c, *_, **__):
+    e.grad = None
+    c.grad = None
+
+
+def _quiesce():
+    torch.cuda.synchronize()
+    gc.collect()
+    torch.cuda.empty_cache()
+    time.sleep(0.2)
+
+
+def _loss_fn(method: str):
+    return baseline if method == "baseline" else functools.partial(linear_cross_entropy, impl=method)
 
 
 def benchmark(methods, test_data, n_iteration, n_rep, dtype, output, kinds, softcap):
+    """Repetition 0 of every data set is a warm-up of one iteration and is not reported (unless n_rep is 0)."""
+    for kind in kinds:
+        if kind not in KINDS:
+            raise ValueError(f"Unknown kind {kind=}")
     torch.set_float32_matmul_precision("high")
-    dtype = getattr(torch, dtype)
-    all_stats = []
+    rows = []
     for name in test_data:
-        gen = data.generator(name)
+        make = data.generator(name)
         for rep in range(n_rep + 1):
-            d = gen(dtype=dtype)
+            reported = rep > 0 or n_rep == 0
+            sample = make(dtype=getattr(torch, dtype))
+            e = sample.embedding.requires_grad_(True)
+            c = sample.classifier.requires_grad_(True)
+            cap = sample.softcap if softcap is None else softcap
             for kind in kinds:
-                e, c, t = d.embedding, d.classifier, d.targets
-                kwargs = {"softcap": softcap if softcap is not None else d.softcap}
-                e.requires_grad_(True)
-                c.requires_grad_(True)
-                if kind == "loss-fw":
-                    pass
-                elif kind in ("loss-bw", "loss-fw-bw"):
-                    kwargs["backward"] = True
-                    kwargs["forward"] = kind == "loss-fw-bw"
-                    kwargs["pre_fn"] = clear_grad_fn
-                else:
-                    raise ValueError(f"Unknown kind {kind=}")
-                for m in methods:
-                    f = baseline if m == "baseline" else functools.partial(linear_cross_entropy, impl=m)
-                    stats = memory.Stats.measure(f, e, c, t, n_iteration=n_iteration if rep > 0 else 1, **kwargs)
-                    if rep > 0 or n_rep == 0:
-                        all_stats.append({"method": m, "kind": kind} | asdict(stats) | {"test_data": name})
-                        torch.cuda.synchronize()
-                        gc.collect()
-                        torch.cuda.empty_cache()
-                        time.sleep(0.2)
-            del d
-    frame = pd.DataFrame(all_stats)
+                fwd, bwd = KINDS[kind]
+                how = dict(forward=fwd, backward=bwd, pre_fn=_drop_grads) if bwd else {}
+                for method in methods:
+                    stats = memory.Stats.measure(_loss_fn(method), e, c, sample.targets, softcap=cap,
+                                                 n_iteration=n_iteration if rep > 0 else 1, **how)
+                    if reported:
+                        rows.append({"method": method, "kind": kind, **dataclasses.asdict(stats), "test_data": name})
+                        _quiesce()
+            del sample, e, c
+    table = pd.DataFrame(rows)
     pd.options.display.float_format = "{:.1f}".format
-    print(frame)
+    print(table)
     if output is not None:
-        path = Path(output)
-        path.parent.mkdir(parents=True, exist_ok=True)
-        frame.to_csv(path)
-    return frame
+        out = pathlib.Path(output)
+        out.parent.mkdir(parents=True, exist_ok=True)
+        table.to_csv(out)
+    return table
+
+
+def _csv(text: str):
+    return [item for item in text.split(",") if item]
 
 
 def main(argv=None):
     ap = argparse.ArgumentParser(prog="python -m benchmark")
-    ap.add_argument("--methods", default="cce,torch_compile,baseline,cce_exact")
-    ap.add_argument("--test_data", default="gemma2")
+    ap.add_argument("--methods", type=_csv, default=_csv("cce,torch_compile,baseline,cce_exact"))
+    ap.add_argument("--test_data", type=_csv, default=_csv("gemma2"))
+    ap.add_argument("--kinds", type=_csv, default=list(KINDS))
     ap.add_argument("--n_iteration", type=int, default=50)
     ap.add_argument("--n_rep", type=int, default=1)
     ap.add_argument("--dtype", default="bfloat16")
-    ap.add_argument("--output", default=None)
-    ap.add_argument("--kinds", default="loss-fw,loss-bw,loss-fw-bw")
     ap.add_argument("--softcap", type=float, default=None)
+    ap.add_argument("--output", default=None)
     a = ap.parse_args(argv)
-    return benchmark(a.methods.split(","), a.test_data.split(","), a.n_iteration, a.n_rep, a.dtype, a.output,
-                     a.kinds.split(","), a.softcap)
+    return benchmark(a.methods, a.test_data, a.n_iteration, a.n_rep, a.dtype, a.output, a.kinds, a.softcap)
 
 
 if __name__ == "__main__":

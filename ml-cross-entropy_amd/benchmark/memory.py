@@ -11,9 +11,23 @@ from typing import Callable, Optional
 
 import torch
 
+_PEAK = "allocated_bytes.all.peak"
 
-def mem_delta(s1, s0) -> int:
-    return s1["allocated_bytes.all.peak"] - s0["allocated_bytes.all.peak"]
+
+class _PeakRise:
+    """Bytes by which the allocator's peak rose since the last ``restart``."""
+
+    def restart(self) -> None:
+        torch.cuda.reset_peak_memory_stats()
+        self._before = torch.cuda.memory_stats()[_PEAK]
+
+    def read(self) -> int:
+        torch.cuda.synchronize()
+        return torch.cuda.memory_stats()[_PEAK] - self._before
+
+
+def _backprop(out: torch.Tensor) -> None:
+    (out if out.numel() == 1 else out.mean()).backward()
 
 
 @dataclass(frozen=True)
@@ -32,45 +46,40 @@ class Stats:
         pre_fn: Optional[Callable[..., None]] = None,
         **kwds,
     ) -> "Stats":
-        if pre_fn is not None:
-            pre_fn(*args, **kwds)
+        def prepare():
+            if pre_fn is not None:
+                pre_fn(*args, **kwds)
+
+        # memory: one call on a quiet allocator
+        prepare()
         torch.cuda.synchronize()
         gc.collect()
         torch.cuda.empty_cache()
-
-        torch.cuda.reset_peak_memory_stats()
-        s0 = torch.cuda.memory_stats()
-        t = f(*args, **kwds)
-        torch.cuda.synchronize()
-        s1 = torch.cuda.memory_stats()
-        if backward and not forward:
-            torch.cuda.reset_peak_memory_stats()
-            s0 = torch.cuda.memory_stats()
+        rise = _PeakRise()
+        rise.restart()
+        out = f(*args, **kwds)
+        mem_bytes = rise.read()
         if backward:
-            if t.numel() > 1:
-                t = t.mean()
-            t.backward()
-            torch.cuda.synchronize()
-            s1 = torch.cuda.memory_stats()
-        mem_bytes = mem_delta(s1, s0)
-
-        events = []
-        for _ in range(n_iteration):
-            if pre_fn is not None:
-                pre_fn(*args, **kwds)
-            start = torch.cuda.Event(enable_timing=True)
-            if forward:
-                start.record(torch.cuda.current_stream())
-            t = f(*args, **kwds)
             if not forward:
-                start.record(torch.cuda.current_stream())
+                rise.restart()
+            _backprop(out)
+            mem_bytes = rise.read()
+
+        # time: device events around the part that was asked for
+        stream = torch.cuda.current_stream()
+        spans = []
+        for _ in range(n_iteration):
+            prepare()
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if forward:
+                begin.record(stream)
+            out = f(*args, **kwds)
+            if not forward:
+                begin.record(stream)
             if backward:
-                if t.numel() > 1:
-                    t = t.mean()
-                t.backward()
-            end = torch.cuda.Event(enable_timing=True)
-            end.record(torch.cuda.current_stream())
-            events.append((start, end))
+                _backprop(out)
+            end.record(stream)
+            spans.append((begin, end))
         torch.cuda.synchronize()
-        total = sum(a.elapsed_time(b) for a, b in events)
-        return cls(total / max(n_iteration, 1), mem_bytes / 2**20)
+        total_ms = sum(b.elapsed_time(e) for b, e in spans)
+        return cls(total_ms / max(n_iteration, 1), mem_bytes / 2**20)

@@ -1,9 +1,12 @@
-"""Autograd glue of the Cut Cross-Entropy loss (reference: cut_cross_entropy/cce.py).
+"""Autograd node of the Cut Cross-Entropy loss on gfx950 (reference: cut_cross_entropy/cce.py).
 
-Forward: fused matmul + log-sum-exp kernel -> gather-dot for the correct-class logit ->
-``nll = lse - correct_logit`` -> reduction.  Backward: one fused kernel that recomputes
-logit tiles and accumulates dE / dC / dBias.  All three kernels are hand-written gfx950
-HIP code behind the C ABI of ``libcce_hip.so``.
+forward    lse[i]  = logsumexp_v softcap(e[row_i] . c[v] + bias[v])      cce_lse_forward   (HIP)
+           dot[i]  = -softcap(e[row_i] . c[t_i] + bias[t_i])            cce_indexed_neg_dot (HIP)
+           nll     = lse + dot, then mean / sum / scatter to the batch shape
+backward   dE, dC, dBias from recomputed logit tiles                    cce_backward / cce_backward_dz (HIP)
+
+fp32 inputs go through ``fp32_path`` (three bf16 parts per value); everything else here is bookkeeping:
+which rows count, where their targets sit, what the upstream gradients mean for each reduction.
 """
 
 from dataclasses import dataclass
@@ -17,35 +20,63 @@ from cut_cross_entropy.cce_backward import cce_backward_kernel
 from cut_cross_entropy.cce_lse_forward import lse_forward
 from cut_cross_entropy.constants import IGNORE_INDEX
 from cut_cross_entropy.indexed_dot import indexed_neg_dot_forward_kernel
-from cut_cross_entropy.utils import (
-    TensorInfo,
-    _build_flat_valids,
-    _handle_eps,
-    handle_reduction_none,
-)
+from cut_cross_entropy.utils import TensorInfo, _build_flat_valids, _handle_eps, handle_reduction_none
 from cut_cross_entropy.vocab_parallel.utils import VocabParallelOptions, require_single_rank
 
+_REDUCTIONS = ("mean", "sum", "none")
 
-@dataclass
+
+@dataclass(frozen=True)
 class CCEParams:
+    """Everything about one call that is not a differentiable tensor (reference: cce.py:26-40)."""
+
+    # which rows of the flattened e enter the loss and where their targets are
     targets: torch.Tensor
     valids: Optional[torch.Tensor]
+    batch_shape: torch.Size
+    shift: int
+    # the loss itself
     softcap: Optional[float]
     reduction: str
+    return_lse: bool
+    # the backward
     filter_eps: Optional[float]
-    shift: int
-    batch_shape: torch.Size
-    accum_e_fp32: bool
-    accum_c_fp32: bool
     filter_e_grad: bool
     filter_c_grad: bool
-    vocab_parallel_options: Optional[VocabParallelOptions]
-    return_lse: bool
+    accum_e_fp32: bool
+    accum_c_fp32: bool
+    vocab_parallel_options: Optional[VocabParallelOptions] = None
+
+    @property
+    def first_class(self) -> int:
+        """Global index of the first class of ``c`` (non-zero for a vocabulary shard)."""
+        vp = self.vocab_parallel_options
+        return 0 if vp is None else vp.start
+
+    def to_batch(self, per_row: torch.Tensor) -> torch.Tensor:
+        """Per-valid-row values laid out in the batch shape, zeros where a target is ignored."""
+        return handle_reduction_none(self.batch_shape, self.valids, self.shift, per_row)
+
+    def reduce(self, nll: torch.Tensor) -> torch.Tensor:
+        if self.reduction == "mean":
+            return nll.mean()  # over the valid rows; NaN when there are none, like F.cross_entropy
+        if self.reduction == "sum":
+            return nll.sum()
+        if self.reduction == "none":
+            return self.to_batch(nll)
+        raise ValueError(f"Unknown reduction {self.reduction}")
+
+    def loss_grad_scale(self, n_valid: int) -> float:
+        """Factor between the upstream gradient of the returned loss and that of a row's nll."""
+        if self.reduction == "mean":
+            return 1.0 / n_valid if n_valid > 0 else 0.0  # no valid row: zero gradients, no exception
+        if self.reduction in ("sum", "none"):
+            return 1.0
+        raise ValueError(f"Unknown reduction {self.reduction}")
 
 
-# Device tensor of uint64[4] that, when set, receives the backward tile counters
-# (tiles in the grid, recomputed, with a dE product, with a dC product).  Used by the
-# benchmark to report the kept-tile fractions of the timed run.
+# uint64[4] device tensor that, while set, accumulates the backward's sub-tile counters (in the plane,
+# recomputed, with a dE product, with a dC product); the benchmark reads the kept fractions from it.
 _tile_counters: Optional[torch.Tensor] = None
 
 
@@ -54,145 +85,95 @@ def set_tile_counters(t: Optional[torch.Tensor]) -> None:
     _tile_counters = t
 
 
+def _autocast_inputs(*tensors):
+    """Inside an autocast region the inputs are taken to the autocast dtype by hand (custom_fwd does not
+    cast when the function is entered with autocast on)."""
+    if not torch.is_autocast_enabled():
+        return tensors
+    low = torch.get_autocast_gpu_dtype()
+    return tuple(t if t is None else t.to(dtype=low) for t in tensors)
+
+
 class LinearCrossEntropyFunction(torch.autograd.Function):
     """Reference: cce.py:48-235."""
 
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, e, c, bias, params: CCEParams):
-        needs_grad = e.requires_grad or c.requires_grad or (bias is not None and bias.requires_grad)
-        # the forward statistic that lets the backward drop tiles is only useful with filtering
-        want_tile_max = needs_grad and params.filter_eps is not None
+        as_given = [None if t is None else TensorInfo(t.dtype, t.requires_grad) for t in (e, c, bias)]
+        any_grad = any(info is not None and info.requires_grad for info in as_given)
+        e, c, bias = _autocast_inputs(e, c, bias)
 
-        e_info = TensorInfo(e.dtype, e.requires_grad)
-        c_info = TensorInfo(c.dtype, c.requires_grad)
-        bias_info = TensorInfo(bias.dtype, bias.requires_grad) if bias is not None else None
-
-        if torch.is_autocast_enabled():
-            low = torch.get_autocast_gpu_dtype()
-            e = e.to(dtype=low)
-            c = c.to(dtype=low)
-            if bias is not None:
-                bias = bias.to(dtype=low)
-
-        vp = params.vocab_parallel_options
-        ctx.fp32 = e.dtype == torch.float32
-        if ctx.fp32:
-            # fp32 values as three bf16 parts along a six times longer reduction axis: fp32_path.py
+        is_fp32 = e.dtype == torch.float32
+        tile_max = None
+        if is_fp32:
             assert c.dtype == torch.float32, "e and c must have the same dtype"
             _hip.require_gpu_tensor("e", e)
             e = e.contiguous()
             lse = fp32_path.fp32_lse(e, c, bias, params.valids, params.softcap)
-            tile_max = None
-            neg_dot = fp32_path.fp32_indexed_neg_dot(
-                e, c, bias, params.targets, params.valids, params.shift, params.softcap,
-                vp.start if vp is not None else 0)
+            neg_dot = fp32_path.fp32_indexed_neg_dot(e, c, bias, params.targets, params.valids, params.shift,
+                                                     params.softcap, params.first_class)
         else:
-            lse, _, tile_max = lse_forward(
-                e, c, bias, params.valids, params.softcap, want_tile_max=want_tile_max
-            )
-            neg_dot = indexed_neg_dot_forward_kernel(
-                e=e,
-                c=c,
-                inds=params.targets,
-                bias=bias,
-                shift=params.shift,
-                valids=params.valids,
-                softcap=params.softcap,
-                out_dtype=lse.dtype,
-                target_offset=vp.start if vp is not None else 0,
-            )
+            # the per-sub-tile maxima let the backward drop sub-tiles unseen; only a filtered backward reads them
+            lse, _, tile_max = lse_forward(e, c, bias, params.valids, params.softcap,
+                                           want_tile_max=any_grad and params.filter_eps is not None)
+            neg_dot = indexed_neg_dot_forward_kernel(e, c, params.targets, bias, params.shift, params.valids,
+                                                     params.softcap, lse.dtype, params.first_class)
         nll = neg_dot.add_(lse)
 
         ctx.save_for_backward(e, c, bias, lse, params.targets, params.valids, tile_max)
-        ctx.params = params
-        ctx.e_info = e_info
-        ctx.c_info = c_info
-        ctx.bias_info = bias_info
-
-        lse_out = None
-        if params.return_lse:
-            lse_out = handle_reduction_none(params.batch_shape, params.valids, params.shift, lse)
-
-        reduction = params.reduction
-        if reduction == "mean":
-            loss = nll.mean()
-        elif reduction == "sum":
-            loss = nll.sum()
-        elif reduction == "none":
-            loss = handle_reduction_none(params.batch_shape, params.valids, params.shift, nll)
-        else:
-            raise ValueError(f"Unknown reduction {reduction}")
-        return loss, lse_out
+        ctx.params, ctx.as_given, ctx.is_fp32 = params, as_given, is_fp32
+        return params.reduce(nll), (params.to_batch(lse) if params.return_lse else None)
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
-    def backward(ctx, grad_out, grad_lse_out):
+    def backward(ctx, d_loss, d_lse):
         e, c, bias, lse, targets, valids, tile_max = ctx.saved_tensors
         params: CCEParams = ctx.params
+        e_info, c_info, bias_info = ctx.as_given
 
-        reduction = params.reduction
-        if reduction == "mean":
-            # zero valid rows: the forward already returned NaN; give zero gradients
-            grad_scale = 1.0 / lse.numel() if lse.numel() > 0 else 0.0
-        elif reduction == "sum":
-            grad_scale = 1.0
-        elif reduction == "none":
-            grad_scale = 1.0
-            grad_out = grad_out.reshape(-1)
-        else:
-            raise ValueError(f"Unknown reduction {reduction}")
-        if grad_lse_out is not None:
-            grad_lse_out = grad_lse_out.reshape(-1)
+        scale = params.loss_grad_scale(lse.numel())
+        # "none": one upstream value per batch position, read by the kernels at row + shift; else one scalar
+        d_loss = d_loss.reshape(-1)
+        if d_lse is not None:
+            d_lse = d_lse.reshape(-1)
 
-        vp = params.vocab_parallel_options
-        if ctx.fp32:
+        if ctx.is_fp32:
             de, dc, dbias = fp32_path.fp32_backward(
-                e, c, bias, lse, grad_out, grad_lse_out, valids, targets, params.shift,
-                vp.start if vp is not None else 0, params.softcap, grad_scale,
-                ctx.e_info.requires_grad, ctx.c_info.requires_grad,
-                ctx.bias_info is not None and ctx.bias_info.requires_grad)
+                e, c, bias, lse, d_loss, d_lse, valids, targets, params.shift, params.first_class, params.softcap,
+                scale, e_info.requires_grad, c_info.requires_grad, bias_info is not None and bias_info.requires_grad)
             if dbias is not None:
-                dbias = dbias.to(ctx.bias_info.dtype)
-            return de, dc, dbias, None
-        de, dc, dbias = cce_backward_kernel(
-            do=grad_out,
-            dlse=grad_lse_out,
-            e=e,
-            e_info=ctx.e_info,
-            c=c,
-            c_info=ctx.c_info,
-            bias=bias,
-            bias_info=ctx.bias_info,
-            lse=lse,
-            valids=valids,
-            softcap=params.softcap,
-            filter_eps=params.filter_eps,
-            targets=targets,
-            shift=params.shift,
-            vocab_ordering=None,
-            grad_scale=grad_scale,
-            accum_e_fp32=params.accum_e_fp32,
-            accum_c_fp32=params.accum_c_fp32,
-            filter_e_grad=params.filter_e_grad,
-            filter_c_grad=params.filter_c_grad,
-            tile_max=tile_max,
-            target_offset=vp.start if vp is not None else 0,
-            counters=_tile_counters,
-        )
+                dbias = dbias.to(bias_info.dtype)
+        else:
+            de, dc, dbias = cce_backward_kernel(
+                d_loss, d_lse, e, e_info, c, c_info, bias, bias_info, lse, valids, params.softcap, params.filter_eps,
+                targets=targets, shift=params.shift, grad_scale=scale,
+                accum_e_fp32=params.accum_e_fp32, accum_c_fp32=params.accum_c_fp32,
+                filter_e_grad=params.filter_e_grad, filter_c_grad=params.filter_c_grad,
+                tile_max=tile_max, target_offset=params.first_class, counters=_tile_counters)
         return de, dc, dbias, None
 
 
 def linear_cross_entropy_apply(e, c, bias, params: CCEParams):
-    """Reference: cce.py:238-256.  The slice after the autograd function makes autograd
-    zero-pad the upstream gradients back to the full batch shape."""
+    """Runs the node and cuts the first ``shift`` positions off batch-shaped outputs (reference:
+    cce.py:238-256); slicing outside the node lets autograd pad the upstream gradients back with zeros."""
     loss, lse = LinearCrossEntropyFunction.apply(e, c, bias, params)
-    if params.shift != 0 and params.reduction == "none":
-        loss = loss[..., params.shift :]
-    if params.return_lse and params.shift != 0:
-        assert lse is not None
-        lse = lse[..., params.shift :]
+    if params.shift:
+        if params.reduction == "none":
+            loss = loss[..., params.shift:]
+        if lse is not None:
+            lse = lse[..., params.shift:]
     return loss, lse
+
+
+def _streamable(c: torch.Tensor) -> bool:
+    """Whether the kernels can stream 16-byte pieces of c's rows where its width allows them to."""
+    per16 = 16 // c.element_size()
+    if c.stride(1) != 1:
+        return False
+    if c.size(1) % per16 != 0:
+        return True  # the element-wise kernels run whatever the layout
+    return c.stride(0) % per16 == 0 and c.data_ptr() % 16 == 0
 
 
 def cce_linear_cross_entropy(
@@ -222,38 +203,31 @@ def cce_linear_cross_entropy(
         )
     if vocab_parallel_options is not None:
         require_single_rank(vocab_parallel_options)
-
-    batch_shape = targets.size()
-    e = e.contiguous()
-    targets = targets.contiguous()
-    # The kernels stream 16-byte pieces of C's rows.  A classifier whose unit stride runs along the classes
-    # (the transpose of a [D, V] matrix), or whose rows start off 16-byte boundaries although D would allow
-    # them not to, takes the element-wise kernels, which are an order of magnitude slower than one packing
-    # copy of C (0.3 ms for 1.2 GB); autograd carries the gradient back through the copy.
-    per16 = 16 // c.element_size()
-    if c.stride(1) != 1 or (c.size(1) % per16 == 0 and (c.stride(0) % per16 != 0 or c.data_ptr() % 16 != 0)):
-        c = c.contiguous()
-
     shift = int(shift)
-    valids = _build_flat_valids(targets, ignore_index, shift)
 
-    e = e.flatten(0, -2)
-    targets = targets.flatten()
-
-    low = torch.get_autocast_gpu_dtype() if torch.is_autocast_enabled() else e.dtype
+    # A classifier whose unit stride runs along the classes (the transpose of a [D, V] matrix), or whose rows
+    # start off 16-byte boundaries although D would allow otherwise, would take the element-wise kernels: an
+    # order of magnitude slower than one packing copy (0.3 ms for 1.2 GB); autograd carries dC back through it.
+    if not _streamable(c):
+        c = c.contiguous()
+    targets = targets.contiguous()
+    compute_dtype = torch.get_autocast_gpu_dtype() if torch.is_autocast_enabled() else e.dtype
+    filtering = filter_eps is not None
     params = CCEParams(
-        targets,
-        valids,
-        softcap,
-        reduction,
-        _handle_eps(filter_eps, low),
-        shift,
-        batch_shape,
-        accum_e_fp32,
-        accum_c_fp32,
-        filter_e_grad=filter_e_grad and filter_eps is not None,
-        filter_c_grad=filter_c_grad and filter_eps is not None,
-        vocab_parallel_options=vocab_parallel_options,
+        targets=targets.flatten(),
+        valids=_build_flat_valids(targets, ignore_index, shift),
+        batch_shape=targets.size(),
+        shift=shift,
+        softcap=softcap,
+        reduction=reduction,
         return_lse=return_lse,
+        filter_eps=_handle_eps(filter_eps, compute_dtype),
+        filter_e_grad=filtering and filter_e_grad,
+        filter_c_grad=filtering and filter_c_grad,
+        accum_e_fp32=accum_e_fp32,
+        accum_c_fp32=accum_c_fp32,
+        vocab_parallel_options=vocab_parallel_options,
     )
-    return linear_cross_entropy_apply(e, c, bias, params)
+    if reduction not in _REDUCTIONS:
+        raise ValueError(f"Unknown reduction {reduction}")
+    return linear_cross_entropy_apply(e.contiguous().flatten(0, -2), c, bias, params)

@@ -52,6 +52,19 @@ def _reject_dtensors(**tensors) -> None:
             raise ValueError(_DTENSOR_MESSAGE.format(name=name))
 
 
+def _check_arguments(c, targets, bias, shift, vocab_parallel_options) -> None:
+    """The argument errors of the reference (linear_cross_entropy.py:131-145), same types and conditions."""
+    steps = targets.size(-1)
+    if isinstance(shift, int) and not 0 <= shift < steps:
+        raise ValueError(f"Shift must be in the range [0, {steps}). Got {shift}.")
+    if vocab_parallel_options is not None:
+        held = vocab_parallel_options.stop - vocab_parallel_options.start
+        if c.size(0) != held:
+            raise ValueError(f"Expected c.size(0) to be {held}, got {c.size(0)}.")
+    if bias is not None and bias.size(0) != c.size(0):
+        raise ValueError(f"Bias has a different number of elements than c. {bias.size(0)} vs. {c.size(0)}.")
+
+
 def linear_cross_entropy(
     e: torch.Tensor,
     c: torch.Tensor,
@@ -72,63 +85,38 @@ def linear_cross_entropy(
 ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
     _reject_dtensors(e=e, c=c, targets=targets, bias=bias)
     impl = impl_name(impl)
+    _check_arguments(c, targets, bias, shift, vocab_parallel_options)
+    common = dict(bias=bias, ignore_index=ignore_index, softcap=softcap, reduction=reduction, shift=shift,
+                  vocab_parallel_options=vocab_parallel_options, return_lse=return_lse)
 
-    if isinstance(shift, int) and (shift < 0 or shift >= targets.size(-1)):
-        raise ValueError(f"Shift must be in the range [0, {targets.size(-1)}). Got {shift}.")
-
-    if vocab_parallel_options is not None:
-        shard = vocab_parallel_options.stop - vocab_parallel_options.start
-        if c.size(0) != shard:
-            raise ValueError(f"Expected c.size(0) to be {shard}, got {c.size(0)}.")
-
-    if bias is not None and bias.size(0) != c.size(0):
-        raise ValueError(
-            f"Bias has a different number of elements than c. {bias.size(0)} vs. {c.size(0)}."
-        )
-
-    if impl in CCEPresets.names:
+    if impl == "torch_compile":
+        loss, lse = torch_compile_linear_cross_entropy(e, c, targets, **common)
+    elif impl in CCEPresets.names:
         if platform.system() == "Darwin":
-            raise RuntimeError(
-                "CCE does not support MacOS. Please use torch_compile when running on MacOS instead."
-            )
-        from cut_cross_entropy.cce import cce_linear_cross_entropy
+            raise RuntimeError("CCE does not support MacOS. Please use torch_compile when running on MacOS instead.")
+        from cut_cross_entropy.cce import cce_linear_cross_entropy  # needs the HIP library: imported on use
 
-        opts = CCEPresets.build_for_impl(
-            impl,
-            CCEPreset(
-                filter_eps=filter_eps,
-                accum_e_fp32=accum_e_fp32,
-                accum_c_fp32=accum_c_fp32,
-                filter_e_grad=filter_e_grad,
-                filter_c_grad=filter_c_grad,
-            ),
-        )
-        loss, lse = cce_linear_cross_entropy(
-            e, c, targets, bias, ignore_index, softcap, reduction, shift,
-            **opts,
-            vocab_parallel_options=vocab_parallel_options,
-            return_lse=return_lse,
-        )
-    elif impl == "torch_compile":
-        loss, lse = torch_compile_linear_cross_entropy(
-            e, c, targets, bias, ignore_index, softcap, reduction, shift,
-            vocab_parallel_options=vocab_parallel_options,
-            return_lse=return_lse,
-        )
+        asked = CCEPreset(filter_eps=filter_eps, accum_e_fp32=accum_e_fp32, accum_c_fp32=accum_c_fp32,
+                          filter_e_grad=filter_e_grad, filter_c_grad=filter_c_grad)
+        loss, lse = cce_linear_cross_entropy(e, c, targets, **common, **CCEPresets.build_for_impl(impl, asked))
     else:
         raise NotImplementedError(f"{impl} is not implemented.")
 
-    if return_lse:
-        assert lse is not None
-        return loss, lse
-    return loss
+    if not return_lse:
+        return loss
+    assert lse is not None
+    return loss, lse
 
 
 linear_cross_entropy.__doc__ = __doc__
 
+_MODULE_OPTIONS = ("ignore_index", "softcap", "reduction", "shift", "filter_eps", "accum_e_fp32", "accum_c_fp32",
+                   "filter_e_grad", "filter_c_grad", "impl", "return_lse")
+
 
 class LinearCrossEntropy(nn.Module):
-    """Module form of :func:`linear_cross_entropy` (reference :201-255)."""
+    """Module form of :func:`linear_cross_entropy` (reference :201-255): the options are fixed at
+    construction and kept as attributes of the same names, the tensors arrive in ``forward``."""
 
     def __init__(
         self,
@@ -145,31 +133,9 @@ class LinearCrossEntropy(nn.Module):
         return_lse: bool = False,
     ):
         super().__init__()
-        self.ignore_index = ignore_index
-        self.softcap = softcap
-        self.reduction = reduction
-        self.shift = shift
-        self.filter_eps = filter_eps
-        self.accum_e_fp32 = accum_e_fp32
-        self.accum_c_fp32 = accum_c_fp32
-        self.filter_e_grad = filter_e_grad
-        self.filter_c_grad = filter_c_grad
-        self.impl = impl
-        self.return_lse = return_lse
+        given = locals()
+        for name in _MODULE_OPTIONS:
+            setattr(self, name, given[name])
 
     def forward(self, e, c, targets, bias=None):
-        return linear_cross_entropy(
-            e, c, targets,
-            bias=bias,
-            ignore_index=self.ignore_index,
-            softcap=self.softcap,
-            reduction=self.reduction,
-            shift=self.shift,
-            filter_eps=self.filter_eps,
-            accum_e_fp32=self.accum_e_fp32,
-            accum_c_fp32=self.accum_c_fp32,
-            filter_e_grad=self.filter_e_grad,
-            filter_c_grad=self.filter_c_grad,
-            impl=self.impl,
-            return_lse=self.return_lse,
-        )
+        return linear_cross_entropy(e, c, targets, bias=bias, **{name: getattr(self, name) for name in _MODULE_OPTIONS})

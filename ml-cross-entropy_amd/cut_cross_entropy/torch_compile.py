@@ -15,45 +15,50 @@ from cut_cross_entropy.utils import _build_flat_valids, handle_reduction_none, s
 from cut_cross_entropy.vocab_parallel.utils import VocabParallelOptions, require_single_rank
 
 
+def _wide_logits(e, c, bias, softcap) -> torch.Tensor:
+    """fp32 copy of the (biased, soft-capped) logits, computed in the input dtype like the reference does."""
+    z = e @ c.T
+    if bias is not None:
+        z = z + bias
+    if softcap is not None:
+        z = softcapping(z, softcap)
+    return z.float()
+
+
+def _reduce(per_row: torch.Tensor, reduction: str) -> torch.Tensor:
+    if reduction == "none":
+        return per_row
+    if reduction == "sum":
+        return per_row.sum()
+    if reduction == "mean":
+        return per_row.mean()
+    raise ValueError(f"Unknown reduction {reduction!r}")
+
+
 def torch_compile_linear_cross_entropy_apply(
     e, c, targets, bias=None, softcap=None, *, ignore_index=IGNORE_INDEX, reduction="mean",
     return_lse=False,
 ):
     """Reference: torch_compile.py:18-49 (run eagerly here)."""
-    logits = e @ c.T
-    if bias is not None:
-        logits = logits + bias
-    if softcap is not None:
-        logits = softcapping(logits, softcap)
-    wide = logits.float()
+    wide = _wide_logits(e, c, bias, softcap)
     if not return_lse:
         return F.cross_entropy(wide, targets, ignore_index=ignore_index, reduction=reduction), None
     lse = torch.logsumexp(wide, dim=-1)
-    loss = F.nll_loss(wide - lse.unsqueeze(-1), targets, ignore_index=ignore_index, reduction=reduction)
-    return loss, lse
+    log_p = wide - lse.unsqueeze(-1)
+    return F.nll_loss(log_p, targets, ignore_index=ignore_index, reduction=reduction), lse
 
 
 def _shard_apply(vp: VocabParallelOptions, e, c, targets, bias, softcap, reduction, return_lse):
-    """One vocabulary shard without the exchange steps
-    (reference: vocab_parallel/vocab_parallel_torch_compile.py:64-134)."""
-    logits = e @ c.T
-    if bias is not None:
-        logits = logits + bias
-    if softcap is not None:
-        logits = softcapping(logits, softcap)
-    wide = logits.float()
+    """One vocabulary shard without the exchange steps (reference:
+    vocab_parallel/vocab_parallel_torch_compile.py:64-134): the shard's log-sum-exp, and the correct logit
+    only for the rows whose target the shard holds."""
+    wide = _wide_logits(e, c, bias, softcap)
     lse = torch.logsumexp(wide, dim=-1)
-    mine = (targets >= vp.start) & (targets < vp.stop)
-    local = torch.where(mine, targets - vp.start, torch.zeros_like(targets))
-    correct = torch.where(mine, wide.gather(1, local.view(-1, 1)).squeeze(1), wide.new_zeros(()))
-    loss = lse - correct
-    if reduction == "mean":
-        loss = loss.mean()
-    elif reduction == "sum":
-        loss = loss.sum()
-    elif reduction != "none":
-        raise ValueError(f"Unknown reduction {reduction!r}")
-    return loss, (lse if return_lse else None)
+    local = targets - vp.start
+    held = (local >= 0) & (local < c.size(0))
+    picked = wide.gather(1, local.clamp(0, c.size(0) - 1).view(-1, 1)).squeeze(1)
+    per_row = lse - picked * held
+    return _reduce(per_row, reduction), (lse if return_lse else None)
 
 
 def torch_compile_linear_cross_entropy(
@@ -71,37 +76,31 @@ def torch_compile_linear_cross_entropy(
     """Reference: torch_compile.py:53-117."""
     assert e.size()[0:-1] == targets.size()
     assert e.size(-1) == c.size(1)
-    batch_shape = targets.size()
-    e = e.contiguous()
-    targets = targets.contiguous()
     shift = int(shift)
+    batch_shape = targets.size()
+    targets = targets.contiguous()
     valids = _build_flat_valids(targets, ignore_index, shift)
 
-    e = e.flatten(0, -2)
-    targets = targets.flatten()
+    rows = e.contiguous().flatten(0, -2)
+    labels = targets.flatten()
     if valids is not None:
-        rows = valids.long()
-        e = e[rows]
-        targets = targets[rows + shift]
+        rows = rows[valids.long()]
+        labels = labels[valids.long() + shift]
 
     if vocab_parallel_options is None:
         loss, lse = torch_compile_linear_cross_entropy_apply(
-            e, c, targets, bias, softcap, ignore_index=ignore_index, reduction=reduction,
-            return_lse=return_lse,
-        )
+            rows, c, labels, bias, softcap, ignore_index=ignore_index, reduction=reduction, return_lse=return_lse)
     else:
         require_single_rank(vocab_parallel_options)
-        loss, lse = _shard_apply(
-            vocab_parallel_options, e, c, targets, bias, softcap, reduction, return_lse
-        )
+        loss, lse = _shard_apply(vocab_parallel_options, rows, c, labels, bias, softcap, reduction, return_lse)
+
+    def to_batch(per_row):
+        full = handle_reduction_none(batch_shape, valids, shift, per_row)
+        return full[..., shift:] if shift else full
 
     if reduction == "none":
-        loss = handle_reduction_none(batch_shape, valids, shift, loss)
-        if shift != 0:
-            loss = loss[..., shift:]
+        loss = to_batch(loss)
     if return_lse:
         assert lse is not None
-        lse = handle_reduction_none(batch_shape, valids, shift, lse)
-        if shift != 0:
-            lse = lse[..., shift:]
+        lse = to_batch(lse)
     return loss, lse

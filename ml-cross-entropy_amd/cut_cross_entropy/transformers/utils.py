@@ -3,7 +3,7 @@
 Restates ref: transformers/utils.py:14-78 (``PatchOptions``, ``apply_lce``).
 """
 
-from dataclasses import dataclass
+import dataclasses
 from typing import Optional, Union
 
 import torch
@@ -11,7 +11,7 @@ import torch
 from cut_cross_entropy.linear_cross_entropy import linear_cross_entropy
 
 
-@dataclass
+@dataclasses.dataclass
 class PatchOptions:
     """What ``cce_patch`` was asked for (ref: transformers/utils.py:19-48)."""
 
@@ -25,23 +25,14 @@ class PatchOptions:
     train_only: bool
 
     def to_kwargs(self) -> dict:
-        return dict(
-            impl=self.impl,
-            reduction=self.reduction,
-            filter_eps=self.filter_eps,
-            accum_e_fp32=self.accum_e_fp32,
-            accum_c_fp32=self.accum_c_fp32,
-            filter_e_grad=self.filter_e_grad,
-            filter_c_grad=self.filter_c_grad,
-        )
+        """The fields that are arguments of ``linear_cross_entropy`` (all but ``train_only``)."""
+        kwargs = dataclasses.asdict(self)
+        del kwargs["train_only"]
+        return kwargs
 
     def use_lce(self, labels: Optional[torch.Tensor], training: bool) -> bool:
-        """The fused loss runs when there are labels, and in eval mode only unless ``train_only``."""
-        if labels is None:
-            return False
-        if not training and self.train_only:
-            return False
-        return True
+        """The fused loss needs labels; with ``train_only`` it is also skipped outside training."""
+        return labels is not None and (training or not self.train_only)
 
 
 def apply_lce(
@@ -59,23 +50,10 @@ def apply_lce(
     divided by that count, as the reference does.  ``softcap`` carries a model's final logit
     soft-capping (Gemma 2) into the fused loss; the reference's patch drops it on this path.
     """
-    num_items_in_batch = loss_kwargs.get("num_items_in_batch", None)
-    cce_kwargs = opts.to_kwargs()
-    if num_items_in_batch is not None and cce_kwargs["reduction"] == "mean":
-        cce_kwargs["reduction"] = "sum"
-    else:
-        num_items_in_batch = None
-
-    loss = linear_cross_entropy(
-        e,
-        c,
-        labels.to(e.device),
-        bias=bias,
-        shift=True,
-        softcap=softcap,
-        **cce_kwargs,
-    )
-
-    if num_items_in_batch is not None:
-        loss = loss / num_items_in_batch
-    return loss
+    kwargs = opts.to_kwargs()
+    denominator = loss_kwargs.get("num_items_in_batch")
+    per_item = denominator is not None and kwargs["reduction"] == "mean"
+    if per_item:
+        kwargs["reduction"] = "sum"
+    loss = linear_cross_entropy(e, c, labels.to(e.device), bias=bias, softcap=softcap, shift=True, **kwargs)
+    return loss / denominator if per_item else loss

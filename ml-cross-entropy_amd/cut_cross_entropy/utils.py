@@ -52,13 +52,13 @@ def _build_flat_valids(
 def handle_reduction_none(
     batch_shape: torch.Size, valids: Optional[torch.Tensor], shift: int, loss: torch.Tensor
 ) -> torch.Tensor:
-    """Scatter per-valid-row values into zeros of the batch shape
+    """Per-valid-row values placed at their batch positions (row + shift), zeros elsewhere
     (reference utils.py:52-61)."""
     if valids is None:
         return loss.view(batch_shape)
-    full = loss.new_zeros((batch_shape.numel(),))
-    full[(valids + shift).long() if shift != 0 else valids.long()] = loss
-    return full.view(batch_shape)
+    out = torch.zeros(batch_shape.numel(), dtype=loss.dtype, device=loss.device)
+    out.index_copy_(0, valids.long() + shift, loss)
+    return out.view(batch_shape)
 
 
 def compute_z_loss(
@@ -68,26 +68,20 @@ def compute_z_loss(
     ignore_index: int = IGNORE_INDEX,
     reduction: str = "mean",
 ) -> torch.Tensor:
-    """Z loss ``lse ** 2`` with ignored tokens masked out; "mean" averages over the
-    tokens that are not ignored (reference utils.py:64-102)."""
-    z_loss = lse.pow(2)
-
+    """Z loss, the square of the log-sum-exp, zero where the (shifted) target is ignored; "mean" is taken
+    over the positions that count (reference utils.py:64-102)."""
+    if reduction not in ("mean", "sum", "none"):
+        raise ValueError(f"Invalid reduction: {reduction}")
+    sq = lse.square()
+    counted = sq.numel()
     if targets is not None:
-        shift = int(shift)
-        if shift != 0:
-            targets = targets[..., shift:]
-        keep = targets != ignore_index
-        z_loss = torch.where(keep, z_loss, 0.0)
-        if reduction == "mean":
-            z_loss = z_loss * (z_loss.numel() / keep.count_nonzero().type_as(z_loss))
-
-    if reduction == "mean":
-        return z_loss.mean()
-    if reduction == "sum":
-        return z_loss.sum()
+        kept = targets[..., int(shift):] != ignore_index
+        sq = sq.masked_fill(~kept, 0.0)
+        counted = kept.sum()
     if reduction == "none":
-        return z_loss
-    raise ValueError(f"Invalid reduction: {reduction}")
+        return sq
+    total = sq.sum()
+    return total / counted if reduction == "mean" else total
 
 
 @dataclass
