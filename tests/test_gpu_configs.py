@@ -419,3 +419,42 @@ def test_backward_with_a_classifier_that_is_a_view(layout, impl):
     assert _rel_err(got_dc.cpu(), co.grad) <= 1e-2
     if layout == "row_gaps":
         assert (base.grad[:, D:] == 0).all()
+
+
+@pytest.mark.parametrize("style", ["flat", "mixed", "peaked"])
+@pytest.mark.parametrize("shape", [(1000, 384, 5000), (256, 2304, 4096), (1024, 128, 8224), (333, 256, 12345),
+                                   (2048, 512, 1000), (96, 1152, 2048)])
+def test_ownership_kernels_at_many_shapes(monkeypatch, shape, style):
+    """The filtered backward pinned to the ownership kernels (no switch to the dense path) on ragged and
+    aligned shapes, 5 % of the rows ignored, for a near-uniform soft-max (only target sub-tiles survive), one
+    where many probabilities sit around eps, and a peaked one: against the dense oracle with the filter rule
+    applied.  A sub-tile whose largest |p - onehot| is within rounding of eps may fall on either side; its
+    entries are then below eps, far inside the tolerance."""
+    import cut_cross_entropy.cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import _build_flat_valids
+
+    monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", None)
+    N, D, V = shape
+    g = torch.Generator().manual_seed(N + D + V)
+    t = torch.randint(0, V, (N,), generator=g)
+    if style == "flat":
+        e = torch.randn((N, D), generator=g)
+        c = torch.randn((V, D), generator=g) * (0.5 / D**0.5)
+    elif style == "mixed":
+        e = torch.randn((N, D), generator=g)
+        c = torch.randn((V, D), generator=g) * (2.0 / D**0.5)
+    else:
+        c = torch.randn((V, D), generator=g) * (2.0 / D) ** 0.5
+        e = 4.0 * c[t] + 0.3 * torch.randn((N, D), generator=g)
+    t[torch.randperm(N, generator=g)[: N // 20]] = IGNORE_INDEX
+    e, c, t = e.to(torch.bfloat16).to(DEV), c.to(torch.bfloat16).to(DEV), t.to(DEV)
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    linear_cross_entropy(ed, cd, t, impl="cce", reduction="sum").backward()
+    valids = _build_flat_valids(t, IGNORE_INDEX, 0)
+    _, de, dc, _ = _oracle_on_gpu(e, c, t.clamp_min(0), valids, torch.ones((N,), device=DEV), None, None,
+                                  filter_eps=2.0**-12)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+    assert (ed.grad[t == IGNORE_INDEX] == 0).all()
