@@ -30,16 +30,20 @@ def _dense_chunk_classes(B: int, V: int, D: int) -> int:
             best, best_fill = vc, fill
     return best
 
-# With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path
-# pays for the whole plane once: measured on MI355X the two cross where about one 128-class cell in
-# seven can hold a probability above filter_eps.  Above this fraction (read off the forward pass's
-# tile statistic, one small reduction and one host read) the backward is run unfiltered; an unfiltered
-# gradient is the exact one, so nothing is lost.  None switches the test off.
-DENSE_WHEN_FLAGGED_ABOVE = 0.12
+# With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path pays for
+# the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
+# statistic can hold a probability above filter_eps for E [8192, 2304] x C [256000, 2304], and at 0.083 for
+# E [16384, 4096] x C [128256, 4096], where a workgroup of the ownership kernels covers D in two slices and
+# recomputes its logits for each.  Above DENSE_WHEN_FLAGGED_ABOVE / slices (the fraction is read off the
+# forward's statistic with one small reduction and one host read) the backward runs unfiltered; an
+# unfiltered gradient is the exact one, so nothing is lost.  None switches the test off.
+DENSE_WHEN_FLAGGED_ABOVE = 0.17
+_OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
 
 def _flagged_fraction(tile_max, lse, B, V, filter_eps) -> float:
-    """Fraction of the 32-row x 128-class cells whose bound exp(max logit - min lse) reaches filter_eps."""
+    """Fraction of the cells of the forward statistic (32 rows x ``STAT_COLS`` classes) whose bound
+    exp(max logit - min lse) reaches filter_eps."""
     import math
 
     ntg, nvc = (B + 31) // 32, (V + _hip.STAT_COLS - 1) // _hip.STAT_COLS
@@ -208,7 +212,7 @@ def cce_backward_kernel(
             and _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad, False, None, False, False)):
         n_valid = valids.size(0) if valids is not None else e.size(0)
         dense = _flagged_fraction(tile_max, lse.to(torch.float32), n_valid, c.size(0), float(filter_eps)) \
-            > DENSE_WHEN_FLAGGED_ABOVE
+            > DENSE_WHEN_FLAGGED_ABOVE / -(-e.size(1) // _OWNERSHIP_SLICE_COLS)
     if dense:
         # every GEMM of the dense path accumulates in fp32 internally and each output element is written
         # once (dC, dBias) or summed in a separate fp32 buffer (dE): no fp32 gradient buffers are needed
