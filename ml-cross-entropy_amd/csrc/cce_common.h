@@ -289,10 +289,15 @@ struct LogitTile {
 // spread over the next two steps, and the first fragments of stage s + 1 are read under the MFMAs
 // of the last step.
 // ---------------------------------------------------------------------------------------------
+// M0 (the LDS address of the load) is a reserved register; naming it in the clobber list is what tells the
+// compiler that the statement changes it, and clang remarks on exactly that.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void lds_dma16(const void* gptr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr)
                : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 constexpr int kDmaBK = 64;
 constexpr int kDmaRowBytes = 128;
