@@ -15,7 +15,13 @@ classifier stays small; chunk log-sum-exps are merged with logaddexp.
 
 Backward: the gradient filter threshold of fp32 is far below anything a soft-max produces, so the
 backward is the unfiltered one: the dz kernel runs on the widened matrices and writes dz as fp32, and
-the two products are fp32 GEMMs on the original matrices.
+the two products are fp32 GEMMs on the original matrices (split-part GEMMs were measured slower than the
+library's fp32 GEMM once the splitting passes are counted: 75 against 117 TFLOP/s).
+
+``torch.set_float32_matmul_precision``: "highest" (the default) takes the six terms above; with "high" or
+"medium" the caller has asked for fast fp32 products (the reference then lets Triton use tf32, 10 mantissa
+bits, cce_lse_forward.py:129-131) and the logits are formed from the three leading terms hi*hi + hi*mid +
+mid*hi (16 bits), half the work; the fp32 GEMMs of the backward follow the same switch inside the library.
 """
 
 from typing import Optional, Tuple
@@ -37,33 +43,43 @@ def split3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     return hi, mid, lo
 
 
-def _padded_width(d: int, has_bias: bool) -> int:
-    w = 6 * d + (3 if has_bias else 0)
+def n_terms() -> int:
+    """Cross terms per product: all six under "highest" float32 matmul precision, the leading three otherwise."""
+    return 6 if torch.get_float32_matmul_precision() == "highest" else 3
+
+
+# which part (0 hi, 1 mid, 2 lo) of e and of c meets in term k; the first three are the 16-bit product
+_E_PARTS = (0, 0, 1, 1, 0, 2)
+_C_PARTS = (0, 1, 0, 1, 2, 0)
+
+
+def _padded_width(d: int, has_bias: bool, terms: int) -> int:
+    w = terms * d + (3 if has_bias else 0)
     return (w + 63) // 64 * 64
 
 
-def widen_e(e: torch.Tensor, has_bias: bool) -> torch.Tensor:
-    """[N, D] fp32 -> [N, Dp] bf16 = [hi hi mid mid hi lo (1 1 1) 0 ...]."""
+def widen_e(e: torch.Tensor, has_bias: bool, terms: int = 6) -> torch.Tensor:
+    """[N, D] fp32 -> [N, Dp] bf16 = [hi hi mid (mid hi lo) (1 1 1) 0 ...]."""
     n, d = e.shape
-    hi, mid, lo = split3(e)
-    out = torch.zeros((n, _padded_width(d, has_bias)), dtype=torch.bfloat16, device=e.device)
-    for k, part in enumerate((hi, hi, mid, mid, hi, lo)):
-        out[:, k * d : (k + 1) * d] = part
+    parts = split3(e)
+    out = torch.zeros((n, _padded_width(d, has_bias, terms)), dtype=torch.bfloat16, device=e.device)
+    for k in range(terms):
+        out[:, k * d : (k + 1) * d] = parts[_E_PARTS[k]]
     if has_bias:
-        out[:, 6 * d : 6 * d + 3] = 1.0
+        out[:, terms * d : terms * d + 3] = 1.0
     return out
 
 
-def widen_c(c: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
-    """[V, D] fp32 (+ [V] bias) -> [V, Dp] bf16 = [hi mid hi mid lo hi (b_hi b_mid b_lo) 0 ...]."""
+def widen_c(c: torch.Tensor, bias: Optional[torch.Tensor], terms: int = 6) -> torch.Tensor:
+    """[V, D] fp32 (+ [V] bias) -> [V, Dp] bf16 = [hi mid hi (mid lo hi) (b_hi b_mid b_lo) 0 ...]."""
     v, d = c.shape
-    hi, mid, lo = split3(c)
-    out = torch.zeros((v, _padded_width(d, bias is not None)), dtype=torch.bfloat16, device=c.device)
-    for k, part in enumerate((hi, mid, hi, mid, lo, hi)):
-        out[:, k * d : (k + 1) * d] = part
+    parts = split3(c)
+    out = torch.zeros((v, _padded_width(d, bias is not None, terms)), dtype=torch.bfloat16, device=c.device)
+    for k in range(terms):
+        out[:, k * d : (k + 1) * d] = parts[_C_PARTS[k]]
     if bias is not None:
         for k, part in enumerate(split3(bias.to(torch.float32))):
-            out[:, 6 * d + k] = part
+            out[:, terms * d + k] = part
     return out
 
 
@@ -73,12 +89,13 @@ def _chunk(v: int, per_class_bytes: int, budget: int) -> int:
 
 def fp32_lse(e, c, bias, valids, softcap) -> torch.Tensor:
     """Log-sum-exp of the valid rows over the whole vocabulary, fp32 accurate."""
-    e6 = widen_e(e, bias is not None)
+    terms = n_terms()
+    e6 = widen_e(e, bias is not None, terms)
     n_valid = valids.numel() if valids is not None else e.size(0)
     lse = torch.full((n_valid,), float("-inf"), dtype=torch.float32, device=e.device)
     vc = _chunk(c.size(0), e6.size(1) * 2, _WIDE_C_BYTES)
     for v0 in range(0, c.size(0), vc):
-        c6 = widen_c(c[v0 : v0 + vc], bias[v0 : v0 + vc] if bias is not None else None)
+        c6 = widen_c(c[v0 : v0 + vc], bias[v0 : v0 + vc] if bias is not None else None, terms)
         part, _, _ = lse_forward(e6, c6, None, valids, softcap)
         lse = torch.logaddexp(lse, part)
     return lse
@@ -117,7 +134,8 @@ def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offs
     dbias = torch.zeros((v,), dtype=torch.float32, device=dev) if want_dbias else None
     if n_valid == 0 or not (want_de or want_dc or want_dbias):
         return de, dc, dbias
-    e6 = widen_e(e, bias is not None)
+    terms = n_terms()
+    e6 = widen_e(e, bias is not None, terms)
     e_rows = e if rows is None else e.index_select(0, rows)
     de_acc = torch.zeros((n_valid, d), dtype=torch.float32, device=dev) if want_de else None
     vc = min(_chunk(v, e6.size(1) * 2, _WIDE_C_BYTES), _chunk(v, n_valid * 4, _DZ_ELEMS * 4))
@@ -131,7 +149,7 @@ def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offs
         ldz = (m + 3) // 4 * 4
         dz = dz_buf[: n_valid * ldz].view(n_valid, ldz)
         c_chunk = c[v0 : v0 + m]
-        c6 = widen_c(c_chunk, bias[v0 : v0 + m] if bias is not None else None)
+        c6 = widen_c(c_chunk, bias[v0 : v0 + m] if bias is not None else None, terms)
         with torch.cuda.device(dev):
             status = lib.cce_backward_dz(
                 e6.data_ptr(), c6.data_ptr(), None,

@@ -308,3 +308,32 @@ def test_fp32_mean_and_lse_and_shard():
     corr = torch.where(inside, logits.gather(1, (t - s0).clamp(0, s1 - s0 - 1).view(-1, 1)).squeeze(1),
                        torch.zeros(300, dtype=torch.float64))
     assert torch.allclose(one.cpu().double(), torch.logsumexp(logits, 1) - corr, atol=2e-5, rtol=0)
+
+
+@pytest.mark.parametrize("softcap", [None, 20.0])
+def test_fp32_inputs_under_fast_matmul_precision(softcap):
+    """``torch.set_float32_matmul_precision("high")`` asks for fast fp32 products (the reference then uses tf32, 10
+    mantissa bits): the logits are formed from three 16-bit terms instead of six and must still be far better than
+    tf32 would be -- 1e-4 on the per-token loss, 2e-3 on the gradients against the fp64 oracle."""
+    from cut_cross_entropy import fp32_path, linear_cross_entropy
+    from oracle import dense_lce
+
+    e, c, t, _ = make_inputs(512, 2000, 256, torch.float32, seed=14, invalid_frac=0.1)
+    el = e.double().requires_grad_(True)
+    cl = c.double().requires_grad_(True)
+    want, _ = dense_lce.dense_linear_cross_entropy(el, cl, t, softcap=softcap, reduction="none")
+    want.sum().backward()
+    before = torch.get_float32_matmul_precision()
+    try:
+        torch.set_float32_matmul_precision("high")
+        assert fp32_path.n_terms() == 3
+        ed = e.cuda().requires_grad_(True)
+        cd = c.cuda().requires_grad_(True)
+        got = linear_cross_entropy(ed, cd, t.cuda(), softcap=softcap, reduction="none")
+        got.sum().backward()
+    finally:
+        torch.set_float32_matmul_precision(before)
+    assert fp32_path.n_terms() == 6
+    assert torch.allclose(got.detach().cpu().double(), want.detach(), atol=1e-4, rtol=0)
+    assert torch.allclose(ed.grad.cpu().double(), el.grad, atol=2e-3, rtol=2e-3)
+    assert torch.allclose(cd.grad.cpu().double(), cl.grad, atol=2e-3, rtol=2e-3)
