@@ -14,12 +14,13 @@
 //             bit is set (all of them when dC is not filtered), four at a time, recomputes the 32 x 32
 //             logits, and accumulates dC^T (D x 32 classes) += E_cell^T . dz; dBias is the row sum of the
 //             same dz.  Rows are written once at the end.
-// Both passes are one kernel template (bwd_owner_kernel) with the roles of E and C swapped.
+// Both passes are one kernel template with the roles of E and C swapped: bwd_owner_kernel for any layout,
+// bwd_owner_fast_kernel (direct-to-LDS loads, D % 128 == 0, 16-byte aligned rows) for the common one.
 //
-// Which sub-blocks can matter: the forward pass left, per 32 rows x 128 classes, the largest
-// soft-capped logit.  If the bound exp(cell_max - min_row lse) of a cell is below filter_eps, every
-// |p| in it is below filter_eps, so only the sub-blocks that hold a target of one of the rows can
-// survive the filter: the others are skipped without being recomputed.
+// Which sub-blocks can matter: the forward pass left, per 32 rows x 32 classes, the largest
+// soft-capped logit.  If the bound exp(cell_max - min_row lse) of a sub-block is below filter_eps, every
+// |p| in it is below filter_eps, so it can survive the filter only if it holds a target of one of the
+// rows: the others are skipped without being recomputed.
 //
 // The price of ownership is that kept sub-tiles are recomputed once more in the second kernel;
 // with filtering that is a small fraction of the plane.  Results are deterministic.
