@@ -85,12 +85,19 @@ def set_tile_counters(t: Optional[torch.Tensor]) -> None:
     _tile_counters = t
 
 
+def _autocast_dtype() -> Optional[torch.dtype]:
+    """The GPU autocast dtype while an autocast region is active, else None."""
+    if hasattr(torch, "get_autocast_dtype"):
+        return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else None
+    return torch.get_autocast_gpu_dtype() if torch.is_autocast_enabled() else None
+
+
 def _autocast_inputs(*tensors):
     """Inside an autocast region the inputs are taken to the autocast dtype by hand (custom_fwd does not
     cast when the function is entered with autocast on)."""
-    if not torch.is_autocast_enabled():
+    low = _autocast_dtype()
+    if low is None:
         return tensors
-    low = torch.get_autocast_gpu_dtype()
     return tuple(t if t is None else t.to(dtype=low) for t in tensors)
 
 
@@ -211,7 +218,7 @@ def cce_linear_cross_entropy(
     if not _streamable(c):
         c = c.contiguous()
     targets = targets.contiguous()
-    compute_dtype = torch.get_autocast_gpu_dtype() if torch.is_autocast_enabled() else e.dtype
+    compute_dtype = _autocast_dtype() or e.dtype
     filtering = filter_eps is not None
     params = CCEParams(
         targets=targets.flatten(),

@@ -337,3 +337,47 @@ def test_fp32_inputs_under_fast_matmul_precision(softcap):
     assert torch.allclose(got.detach().cpu().double(), want.detach(), atol=1e-4, rtol=0)
     assert torch.allclose(ed.grad.cpu().double(), el.grad, atol=2e-3, rtol=2e-3)
     assert torch.allclose(cd.grad.cpu().double(), cl.grad, atol=2e-3, rtol=2e-3)
+
+
+@pytest.mark.parametrize("ignore_index", [0, 7, 10**6])
+def test_custom_ignore_index(ignore_index):
+    """An ignore value that is itself a class index (or far outside the vocabulary): those rows drop out of loss
+    and gradients, every other row is unaffected (reference: the ignore_index argument, cce.py:286-290)."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    e, c, t, _ = make_inputs(300, 500, 64, torch.bfloat16, seed=15)
+    t[::5] = ignore_index
+    el, cl = e.double().requires_grad_(True), c.double().requires_grad_(True)
+    want, _ = dense_lce.dense_linear_cross_entropy(el, cl, t, ignore_index=ignore_index)
+    want.backward()
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    got = linear_cross_entropy(ed, cd, t.cuda(), ignore_index=ignore_index, impl="cce_exact")
+    got.backward()
+    assert abs(got.item() - want.item()) <= 1e-3 * abs(want.item())
+    assert (ed.grad.cpu()[t == ignore_index] == 0).all()
+    assert torch.allclose(ed.grad.cpu().double(), el.grad, atol=1e-2 / 240, rtol=2e-2)
+    assert torch.allclose(cd.grad.cpu().double(), cl.grad, atol=1e-2 / 240, rtol=2e-2)
+
+
+@pytest.mark.parametrize("low", [torch.bfloat16, torch.float16])
+def test_autocast_region(low):
+    """fp32 parameters inside ``torch.autocast``: the kernels run in the autocast dtype, the loss is fp32 and the
+    gradients come back in the dtype of the leaves (reference: custom_fwd / custom_bwd and the manual cast,
+    cce.py:50,71-76,165)."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    e, c, t, _ = make_inputs(256, 700, 128, torch.float32, seed=16)
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    with torch.autocast(device_type="cuda", dtype=low):
+        loss = linear_cross_entropy(ed, cd, t.cuda(), impl="cce_exact")
+    loss.backward()
+    assert loss.dtype == torch.float32 and ed.grad.dtype == torch.float32 and cd.grad.dtype == torch.float32
+    el, cl = e.to(low).double().requires_grad_(True), c.to(low).double().requires_grad_(True)
+    want, _ = dense_lce.dense_linear_cross_entropy(el, cl, t)
+    want.backward()
+    tol = 1e-2 if low == torch.bfloat16 else 2e-3
+    assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+    assert torch.allclose(ed.grad.cpu().double(), el.grad, atol=tol / 256, rtol=2 * tol)
+    assert torch.allclose(cd.grad.cpu().double(), cl.grad, atol=tol / 256, rtol=2 * tol)
