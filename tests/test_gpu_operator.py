@@ -381,3 +381,29 @@ def test_autocast_region(low):
     assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
     assert torch.allclose(ed.grad.cpu().double(), el.grad, atol=tol / 256, rtol=2 * tol)
     assert torch.allclose(cd.grad.cpu().double(), cl.grad, atol=tol / 256, rtol=2 * tol)
+
+
+def test_int32_targets_and_strided_embeddings():
+    """Targets as int32 and embeddings that are a strided view of a wider activation tensor, batch shape
+    [2, 3, T]: same loss as with int64 targets and a packed copy, gradients arrive in the view's base."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    e, c, t, _ = make_inputs(6 * 40, 300, 64, torch.bfloat16, seed=17, invalid_frac=0.1)
+    base = torch.zeros((2, 3, 40, 96), dtype=torch.bfloat16, device="cuda")
+    base[..., :64] = e.view(2, 3, 40, 64).cuda()
+    base.requires_grad_(True)
+    view = base[..., :64]
+    assert not view.is_contiguous()
+    cd = c.cuda().requires_grad_(True)
+    t3 = t.view(2, 3, 40).cuda()
+    got = linear_cross_entropy(view, cd, t3.to(torch.int32), reduction="none", shift=1, impl="cce_exact")
+    assert got.shape == (2, 3, 39)
+    got.sum().backward()
+    g_view, g_c = base.grad[..., :64].clone(), cd.grad.clone()
+    assert (base.grad[..., 64:] == 0).all()
+
+    packed = view.detach().contiguous().requires_grad_(True)
+    cd.grad = None
+    want = linear_cross_entropy(packed, cd, t3, reduction="none", shift=1, impl="cce_exact")
+    want.sum().backward()
+    assert torch.equal(got, want) and torch.equal(g_view, packed.grad) and torch.equal(g_c, cd.grad)
