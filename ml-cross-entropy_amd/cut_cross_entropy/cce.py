@@ -183,6 +183,7 @@ def _streamable(c: torch.Tensor) -> bool:
     return c.stride(0) % per16 == 0 and c.data_ptr() % 16 == 0
 
 
+@torch.compiler.disable  # ctypes launches and a host read of the valid rows: a graph break for torch.compile, not a trace
 def cce_linear_cross_entropy(
     e: torch.Tensor,
     c: torch.Tensor,

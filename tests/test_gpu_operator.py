@@ -407,3 +407,25 @@ def test_int32_targets_and_strided_embeddings():
     want = linear_cross_entropy(packed, cd, t3, reduction="none", shift=1, impl="cce_exact")
     want.sum().backward()
     assert torch.equal(got, want) and torch.equal(g_view, packed.grad) and torch.equal(g_c, cd.grad)
+
+
+def test_inside_a_compiled_function():
+    """Called from a function under ``torch.compile`` the operator is a graph break (it launches through ctypes
+    and reads the number of valid rows on the host), not a tracing error; values and gradients equal eager."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    e, c, t, _ = make_inputs(128, 300, 64, torch.bfloat16, seed=18, invalid_frac=0.1)
+    td = t.cuda()
+
+    def fn(x, w):
+        return linear_cross_entropy(x * 2.0, w, td, softcap=10.0, impl="cce_exact") * 0.5
+
+    outs = []
+    for f in (fn, torch.compile(fn, backend="aot_eager")):
+        x = e.cuda().requires_grad_(True)
+        w = c.cuda().requires_grad_(True)
+        loss = f(x, w)
+        loss.backward()
+        outs.append((loss.detach(), x.grad, w.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
