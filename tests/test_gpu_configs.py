@@ -458,3 +458,112 @@ def test_ownership_kernels_at_many_shapes(monkeypatch, shape, style):
     assert _rel_err(ed.grad, de) <= 1e-2
     assert _rel_err(cd.grad, dc) <= 1e-2
     assert (ed.grad[t == IGNORE_INDEX] == 0).all()
+
+
+def test_config5_full_size_filtered():
+    """E [65536, 3584] peaked on its labels, C [152064, 3584], full vocabulary, gradient filter on: the largest
+    configuration at its real size against the dense oracle with the filter rule, evaluated with torch on the
+    GPU in row chunks; and the fraction of the plane the backward had to look at."""
+    from cut_cross_entropy import cce as cce_mod
+    from cut_cross_entropy import linear_cross_entropy
+
+    N, D, V = 65536, 3584, 152064
+    g = torch.Generator(device=DEV).manual_seed(5)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (N,), generator=g, device=DEV)
+    e = (4.0 * c[t].float() + 0.5 * torch.randn((N, D), generator=g, device=DEV)).to(torch.bfloat16)
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    counters = torch.zeros(4, dtype=torch.int64, device=DEV)
+    cce_mod.set_tile_counters(counters)
+    loss, lse = linear_cross_entropy(ed, cd, t, impl="cce", return_lse=True)
+    loss.backward()
+    torch.cuda.synchronize()
+    cce_mod.set_tile_counters(None)
+
+    d_out = torch.full((N,), 1.0 / N, device=DEV)
+    want_lse, de, dc, _ = _oracle_on_gpu(e, c, t, None, d_out, None, None, filter_eps=2.0**-12)
+    assert torch.allclose(lse, want_lse, rtol=1e-3, atol=1e-3)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
+    total, recomputed, with_de, with_dc = counters.tolist()
+    assert total == (N // 32) * (V // 32)
+    assert recomputed / total < 0.02 and with_dc == with_de
+
+
+def test_config3_full_size_shift_and_trailing_ignored():
+    """E [4, 4096, 4096], C [128256, 4096], labels with the last 256 of every sequence ignored, shift=1, mean,
+    impl="cce", at full size against the dense oracle evaluated with torch on the GPU."""
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import _build_flat_valids
+    from oracle import dense_lce
+
+    Bt, T, D, V = 4, 4096, 4096, 128256
+    g = torch.Generator(device=DEV).manual_seed(3)
+    e = torch.randn((Bt, T, D), generator=g, device=DEV).to(torch.bfloat16)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (Bt, T), generator=g, device=DEV)
+    t[:, -256:] = IGNORE_INDEX
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    loss, lse = linear_cross_entropy(ed, cd, t, shift=1, impl="cce", return_lse=True)
+    loss.backward()
+
+    valids = _build_flat_valids(t, IGNORE_INDEX, 1)
+    assert valids.numel() == Bt * (T - 256 - 1)  # 15356: the last position of a sequence has no next token
+    flat_t = t.flatten().clamp_min(0)
+    d_out = torch.full((Bt * T,), 1.0 / valids.numel(), device=DEV)
+    # the backward may run filtered or, where most cells can hold a probability above eps, unfiltered
+    want_lse, de_f, dc_f, _ = _oracle_on_gpu(e.view(-1, D), c, flat_t, valids, d_out, None, None, shift=1,
+                                             filter_eps=2.0**-12)
+    _, de_x, dc_x, _ = _oracle_on_gpu(e.view(-1, D), c, flat_t, valids, d_out, None, None, shift=1)
+    assert lse.shape == (Bt, T - 1)
+    full_lse = torch.zeros((Bt * T,), device=DEV)
+    full_lse[valids.long() + 1] = want_lse  # batch-shaped, zeros at ignored positions, first position cut off
+    assert torch.allclose(lse, full_lse.view(Bt, T)[:, 1:], rtol=1e-3, atol=1e-3)
+    nd = dense_lce.dense_indexed_neg_dot(e.view(-1, D)[valids.long()], c, flat_t[valids.long() + 1], None, None,
+                                         torch.float32)
+    want_loss = (want_lse + nd).mean()
+    assert abs(loss.item() - want_loss.item()) <= 1e-3 * abs(want_loss.item())
+    g_e = ed.grad.view(-1, D)
+    assert min(_rel_err(g_e, de_f), _rel_err(g_e, de_x)) <= 1e-2
+    assert min(_rel_err(cd.grad, dc_f), _rel_err(cd.grad, dc_x)) <= 1e-2
+    dead = torch.ones((Bt, T), dtype=torch.bool, device=DEV)
+    dead[:, : T - 1] = t[:, 1:] == IGNORE_INDEX
+    assert (ed.grad[dead] == 0).all()
+
+
+def test_config4_full_size_kahan_full_zloss_none():
+    """E [8192, 2048], C [256000, 2048], Zipf(1.1) labels, impl="cce_kahan_full_c_full_e", reduction none with
+    the z-loss of the returned log-sum-exp (weight 1e-4): per-token loss, log-sum-exp and gradients at full size
+    against the dense oracle evaluated with torch on the GPU."""
+    from cut_cross_entropy import linear_cross_entropy
+    from cut_cross_entropy.utils import compute_z_loss
+    from oracle import dense_lce
+
+    N, D, V, w = 8192, 2048, 256000, 1e-4
+    g = torch.Generator(device=DEV).manual_seed(4)
+    e = torch.randn((N, D), generator=g, device=DEV).to(torch.bfloat16)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    ranks = torch.arange(1, V + 1, dtype=torch.float64, device=DEV)
+    cdf = torch.cumsum(ranks.pow(-1.1), 0)
+    cdf /= cdf[-1].clone()
+    t = torch.searchsorted(cdf, torch.rand(N, generator=g, dtype=torch.float64, device=DEV)).clamp_max(V - 1)
+    assert (t < 100).float().mean() > 0.3  # heavy head: many rows share a class group
+
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    loss, lse = linear_cross_entropy(ed, cd, t, impl="cce_kahan_full_c_full_e", reduction="none", return_lse=True)
+    (loss.mean() + w * compute_z_loss(lse, t)).backward()
+
+    # d/d nll_i = 1 / N; d/d lse_i = w * 2 lse_i / N
+    d_out = torch.full((N,), 1.0 / N, device=DEV)
+    want_lse = torch.cat([dense_lce.dense_lse(e[r], c, None, None, torch.float32)
+                          for r in torch.arange(N, device=DEV).split(2048)])
+    d_lse = w * 2.0 * want_lse / N
+    _, de, dc, _ = _oracle_on_gpu(e, c, t, None, d_out, d_lse, None)
+    want = want_lse + dense_lce.dense_indexed_neg_dot(e, c, t, None, None, torch.float32)
+    assert torch.allclose(lse, want_lse, rtol=1e-3, atol=1e-3)
+    assert torch.allclose(loss, want, rtol=1e-3, atol=1e-3)
+    assert _rel_err(ed.grad, de) <= 1e-2
+    assert _rel_err(cd.grad, dc) <= 1e-2
