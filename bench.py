@@ -105,6 +105,9 @@ def main():
         print("bench.py: this build runs on exactly one GPU (no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()  # loads the library built in the tree; builds it only if there is none
     import torch
 
     from cut_cross_entropy import _hip, linear_cross_entropy

@@ -9,6 +9,13 @@ for p in (ROOT, os.path.join(ROOT, "ml-cross-entropy_amd")):
         sys.path.insert(0, p)
 
 
+def pytest_sessionstart(session):
+    """The tests load the library that is built in the tree; a tree without one gets it built first."""
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real AMD GPU (run with -m gpu on the MI355X box)")
 
