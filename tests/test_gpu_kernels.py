@@ -233,3 +233,51 @@ def test_backward_dz_rejects_layouts_it_cannot_stream():
                              t.data_ptr(), dz.data_ptr(), 128, 0, 64, 64, 128, 72, 72, 72, 1, 1.0, 0, 0, 0.0, 0,
                              torch.cuda.current_stream().cuda_stream)
     assert st == 10004  # CCE_ERR_MISALIGNED
+
+
+def test_entry_points_reject_bad_arguments_before_launching():
+    """Status codes of the C ABI for arguments it cannot run: nothing is launched, outputs stay untouched."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D = 64, 128, 64
+    e = torch.zeros((N, D), dtype=torch.bfloat16, device=dev)
+    c = torch.zeros((V, D), dtype=torch.bfloat16, device=dev)
+    lse = torch.full((N,), 3.0, device=dev)
+    ws = torch.zeros((lib.cce_lse_forward_workspace_bytes(N, V, D) // 8 + 2,), dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    INVALID, DTYPE, WORKSPACE, MISALIGNED = 10001, 10002, 10003, 10004
+
+    def fwd(e_ptr=e.data_ptr(), c_ptr=c.data_ptr(), lse_ptr=lse.data_ptr(), ws_ptr=ws.data_ptr(), ws_bytes=ws.numel() * 8,
+            n=N, b=N, v=V, d=D, dtype=0):
+        return lib.cce_lse_forward(e_ptr, c_ptr, None, None, lse_ptr, None, None, ws_ptr, ws_bytes, n, b, v, d,
+                                   D, D, 1, 0.0, dtype, stream)
+
+    assert fwd() == 0
+    lse.fill_(3.0)
+    assert fwd(b=-1) == INVALID and fwd(v=0) == INVALID and fwd(d=0) == INVALID
+    assert fwd(b=N + 1) == INVALID  # more rows than e holds and no index vector
+    assert fwd(e_ptr=None) == INVALID and fwd(c_ptr=None) == INVALID and fwd(lse_ptr=None) == INVALID
+    assert fwd(dtype=7) == DTYPE
+    assert fwd(ws_ptr=None) == WORKSPACE and fwd(ws_bytes=8) == WORKSPACE
+    assert fwd(ws_ptr=ws.data_ptr() + 4) == MISALIGNED
+    assert fwd(b=0) == 0  # nothing to do is not an error
+    torch.cuda.synchronize()
+    assert (lse == 3.0).all()
+
+    t = torch.zeros((N,), dtype=torch.int64, device=dev)
+    de = torch.zeros((N, D), dtype=torch.bfloat16, device=dev)
+    bws = torch.zeros((lib.cce_backward_workspace_bytes(N, V, D) // 8 + 2,), dtype=torch.int64, device=dev)
+
+    def bwd(lse_ptr=lse.data_ptr(), t_ptr=t.data_ptr(), v=V, shift=0, dtype=0, ws_bytes=bws.numel() * 8, dc_ptr=None):
+        return lib.cce_backward(e.data_ptr(), c.data_ptr(), None, lse_ptr, lse.data_ptr(), 0, None, None, None, t_ptr,
+                                None, de.data_ptr(), dc_ptr, None, bws.data_ptr(), ws_bytes, None,
+                                N, N, v, D, D, D, 1, 1.0, 2.0**-12, 1, 1, 0, 0, shift, 0, 0.0, dtype, stream)
+
+    assert bwd(lse_ptr=None) == INVALID and bwd(t_ptr=None) == INVALID and bwd(shift=-1) == INVALID
+    assert bwd(v=2**31) == INVALID
+    assert bwd(dtype=5) == DTYPE
+    dc = torch.zeros((V, D), dtype=torch.bfloat16, device=dev)
+    assert bwd(dc_ptr=dc.data_ptr(), ws_bytes=0) == WORKSPACE  # a filtered dC needs the survivor bits
+    torch.cuda.synchronize()
+    assert (de == 0).all() and (dc == 0).all()
+    assert lib.cce_error_string(INVALID) and lib.cce_error_string(MISALIGNED) and lib.cce_error_string(DTYPE)
