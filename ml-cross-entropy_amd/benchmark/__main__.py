@@ -54,7 +54,23 @@ def benchmark(methods, test_data, n_iteration, n_rep, dtype, output, kinds, soft
     for kind in kinds:
         if kind not in KINDS:
             raise ValueError(f"Unknown kind {kind=}")
-    torch.set_float32_matmul_precision("high")
+    precision_before = torch.get_float32_matmul_precision()
+    torch.set_float32_matmul_precision("high")  # as the reference's benchmark does (benchmark/__main__.py:52)
+    try:
+        rows = _measure_all(methods, test_data, n_iteration, n_rep, dtype, kinds, softcap)
+    finally:
+        torch.set_float32_matmul_precision(precision_before)
+    table = pd.DataFrame(rows)
+    pd.options.display.float_format = "{:.1f}".format
+    print(table)
+    if output is not None:
+        out = pathlib.Path(output)
+        out.parent.mkdir(parents=True, exist_ok=True)
+        table.to_csv(out)
+    return table
+
+
+def _measure_all(methods, test_data, n_iteration, n_rep, dtype, kinds, softcap):
     rows = []
     for name in test_data:
         make = data.generator(name)
@@ -74,14 +90,7 @@ def benchmark(methods, test_data, n_iteration, n_rep, dtype, output, kinds, soft
                         rows.append({"method": method, "kind": kind, **dataclasses.asdict(stats), "test_data": name})
                         _quiesce()
             del sample, e, c
-    table = pd.DataFrame(rows)
-    pd.options.display.float_format = "{:.1f}".format
-    print(table)
-    if output is not None:
-        out = pathlib.Path(output)
-        out.parent.mkdir(parents=True, exist_ok=True)
-        table.to_csv(out)
-    return table
+    return rows
 
 
 def _csv(text: str):
