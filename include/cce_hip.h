@@ -35,6 +35,7 @@ extern "C" {
 #define CCE_ERR_UNSUPPORTED_DTYPE 10002
 #define CCE_ERR_WORKSPACE_TOO_SMALL 10003
 #define CCE_ERR_MISALIGNED 10004
+#define CCE_ERR_STATIC_SCRATCH_LIMIT 10005
 
 #define CCE_DTYPE_BF16 0
 #define CCE_DTYPE_F16 1
@@ -79,6 +80,28 @@ int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_
                     int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
                     float softcap, int dtype, void* stream);
 
+/* Size of the per-GPU static scratch array behind cce_lse_forward_static. */
+#define CCE_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+
+/*
+ * cce_lse_forward without a workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference, whose launcher allocates its outputs and locks with torch on every
+ * call (cut_cross_entropy/cce_lse_forward.py:193-204).  Same arguments, results and kernels as
+ * cce_lse_forward; the split-vocabulary partials go to a static device array of
+ * CCE_STATIC_SCRATCH_BYTES that each GPU the library runs on holds until the process ends.  The call
+ * allocates and frees nothing.  Shapes whose cce_lse_forward_workspace_bytes() exceeds the array
+ * return CCE_ERR_STATIC_SCRATCH_LIMIT (c2 needs 0.5 MB, E [65536, 3584] x C [152064, 3584] 2 MB).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU race; calls on one
+ * stream, or otherwise ordered, are safe (a launch writes every partial before reading it, so nothing
+ * carries over from the previous call).
+ */
+int cce_lse_forward_static(const void* e, const void* c, const void* bias, const int32_t* valids,
+                           float* lse, float* logit_avg, float* tile_max,
+                           int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                           int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                           float softcap, int dtype, void* stream);
+
 /*
  * out[i] = softcap(-(e[valids[i]] . c[t_i]) - bias[t_i]),  t_i = targets[valids[i] + shift] - target_offset;
  * out[i] = 0 when t_i is outside [0, v).
@@ -92,7 +115,8 @@ int cce_indexed_neg_dot(const void* e, const void* c, const int64_t* targets, co
                         int64_t shift, int64_t target_offset,
                         float softcap, int dtype, void* stream);
 
-/* Scratch bytes cce_backward needs (kept-tile list and its cursor). */
+/* Scratch bytes cce_backward needs: one survivor bit per 32 x 32 sub-tile, each 32-row group's bits
+ * padded to whole 32-bit words. */
 int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d);
 
 /*
@@ -103,8 +127,9 @@ int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d);
  *     dz = (p (g + h) - y g) (1 - (s / softcap)^2)
  *     d_e[row_i] += sum_v dz c[v];  d_c[v] += sum_i dz e[row_i];  d_bias[v] += sum_i dz.
  * A tile of the (row, class) plane whose every |p - y| is below filter_eps is dropped
- * from d_e when filter_e, from d_c when filter_c, and from d_bias when both are set
- * (gradient filtering, reference :211-216).  filter_eps < 0 switches filtering off.
+ * from d_e when filter_e, and from d_c and d_bias when filter_c (gradient filtering,
+ * reference :211-216; the reference drops a tile from d_bias only when both flags are set, the
+ * difference lies within what filtering is allowed to drop).  filter_eps < 0 switches filtering off.
  *
  *   lse        [b] float      (the global LSE when c is a vocabulary shard)
  *   d_out      [n_rows] float read at (row + shift), or one float when d_out_is_scalar

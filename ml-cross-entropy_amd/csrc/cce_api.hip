@@ -1,7 +1,7 @@
 // Version and status text of the C ABI.
 #include "cce_common.h"
 
-extern "C" int cce_version(void) { return 3; }
+extern "C" int cce_version(void) { return 4; }
 
 extern "C" const char* cce_error_string(int status) {
   switch (status) {
@@ -10,6 +10,9 @@ extern "C" const char* cce_error_string(int status) {
     case CCE_ERR_UNSUPPORTED_DTYPE: return "cce: unsupported element type (bf16 and fp16 only)";
     case CCE_ERR_WORKSPACE_TOO_SMALL: return "cce: workspace missing or too small";
     case CCE_ERR_MISALIGNED: return "cce: pointer not aligned as required";
+    case CCE_ERR_STATIC_SCRATCH_LIMIT:
+      return "cce: shape needs more scratch than the static array holds (CCE_STATIC_SCRATCH_BYTES); "
+             "use the entry point that takes a workspace";
     default: return hipGetErrorString(static_cast<hipError_t>(status));
   }
 }

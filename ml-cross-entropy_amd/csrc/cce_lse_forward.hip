@@ -12,6 +12,8 @@
 // into (xcd, slot) and items are numbered so that one XCD works on neighbouring spans of the
 // same few row blocks: its L2 then serves each E block to several workgroups and each C tile to
 // several row blocks.
+#include <atomic>
+
 #include "cce_common.h"
 
 namespace cce {
@@ -359,19 +361,12 @@ extern "C" int64_t cce_lse_forward_workspace_bytes(int64_t b, int64_t v, int64_t
   return static_cast<int64_t>(nsplit) * b * static_cast<int64_t>(sizeof(float2));
 }
 
-extern "C" int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_t* valids,
-                               float* lse, float* logit_avg, float* tile_max,
-                               void* workspace, int64_t workspace_bytes,
-                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
-                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
-                               float softcap, int dtype, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  if (b < 0 || v <= 0 || d <= 0 || n_rows < 0) return CCE_ERR_INVALID_ARGUMENT;
-  if (b == 0) return CCE_OK;
-  if (e == nullptr || c == nullptr || lse == nullptr) return CCE_ERR_INVALID_ARGUMENT;
-  if (valids == nullptr && b > n_rows) return CCE_ERR_INVALID_ARGUMENT;
-  if (d > (1 << 30) || b > (int64_t(1) << 40) || v > (int64_t(1) << 31) - 512) return CCE_ERR_INVALID_ARGUMENT;
-  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+static int lse_forward_impl(const void* e, const void* c, const void* bias, const int32_t* valids,
+                            float* lse, float* logit_avg, float* tile_max,
+                            void* workspace, int64_t workspace_bytes,
+                            int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                            int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                            float softcap, int dtype, hipStream_t stream) {
   const int64_t need = cce_lse_forward_workspace_bytes(b, v, d);
   if (workspace == nullptr || workspace_bytes < need) return CCE_ERR_WORKSPACE_TOO_SMALL;
   if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return CCE_ERR_MISALIGNED;
@@ -411,4 +406,81 @@ extern "C" int cce_lse_forward(const void* e, const void* c, const void* bias, c
   hipLaunchKernelGGL(lse_merge_kernel, dim3(static_cast<unsigned>((b + 255) / 256)), dim3(256), 0, stream,
                      p.partial, lse, b, p.nsplit);
   return status_from_hip(hipGetLastError());
+}
+
+// Argument checks shared by the two entry points; CCE_OK with *done set means "nothing to do".
+static int lse_forward_check(const void* e, const void* c, const float* lse, const int32_t* valids,
+                             int64_t n_rows, int64_t b, int64_t v, int64_t d, int dtype, bool* done) {
+  *done = false;
+  if (b < 0 || v <= 0 || d <= 0 || n_rows < 0) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0) {
+    *done = true;
+    return CCE_OK;
+  }
+  if (e == nullptr || c == nullptr || lse == nullptr) return CCE_ERR_INVALID_ARGUMENT;
+  if (valids == nullptr && b > n_rows) return CCE_ERR_INVALID_ARGUMENT;
+  if (d > (1 << 30) || b > (int64_t(1) << 40) || v > (int64_t(1) << 31) - 512) return CCE_ERR_INVALID_ARGUMENT;
+  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+  return CCE_OK;
+}
+
+extern "C" int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_t* valids,
+                               float* lse, float* logit_avg, float* tile_max,
+                               void* workspace, int64_t workspace_bytes,
+                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                               float softcap, int dtype, void* stream_) {
+  bool done;
+  const int st = lse_forward_check(e, c, lse, valids, n_rows, b, v, d, dtype, &done);
+  if (st != CCE_OK || done) return st;
+  return lse_forward_impl(e, c, bias, valids, lse, logit_avg, tile_max, workspace, workspace_bytes, n_rows, b, v, d,
+                          stride_e, stride_cv, stride_cd, softcap, dtype, static_cast<hipStream_t>(stream_));
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same forward for callers that may not allocate: the split-vocabulary partials live in a
+// file-scope device array instead of a caller's workspace.  Each GPU holds its own copy of the
+// array, at its own address, until the process ends; the address is looked up once per device (with
+// that device current) and from then on only that pointer is used -- the array's name is a host-side
+// handle, not a device address.  Every (span, row) partial a launch reads is written by the same
+// launch first, so nothing has to be cleared between calls; calls that overlap on one GPU (two
+// streams, two threads) share the array and race.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[CCE_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+static int static_scratch_for_current_device(void** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return status_from_hip(err);
+  if (dev < 0 || dev >= kMaxDevices) return CCE_ERR_INVALID_ARGUMENT;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return status_from_hip(err);
+    if (ptr == nullptr) return CCE_ERR_INVALID_ARGUMENT;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = ptr;
+  return CCE_OK;
+}
+
+extern "C" int cce_lse_forward_static(const void* e, const void* c, const void* bias, const int32_t* valids,
+                                      float* lse, float* logit_avg, float* tile_max,
+                                      int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                                      int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                                      float softcap, int dtype, void* stream_) {
+  bool done;
+  int st = lse_forward_check(e, c, lse, valids, n_rows, b, v, d, dtype, &done);
+  if (st != CCE_OK || done) return st;
+  if (cce_lse_forward_workspace_bytes(b, v, d) > CCE_STATIC_SCRATCH_BYTES) return CCE_ERR_STATIC_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  st = static_scratch_for_current_device(&ws);
+  if (st != CCE_OK) return st;
+  return lse_forward_impl(e, c, bias, valids, lse, logit_avg, tile_max, ws, CCE_STATIC_SCRATCH_BYTES, n_rows, b, v, d,
+                          stride_e, stride_cv, stride_cd, softcap, dtype, static_cast<hipStream_t>(stream_));
 }

@@ -16,11 +16,12 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
 STAT_ROWS = 32
 STAT_COLS = 32
 NUM_COUNTERS = 4
+STATIC_SCRATCH_BYTES = 8 * 1024 * 1024
 
 _i64, _i32, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 
@@ -33,6 +34,11 @@ _SIGNATURES = {
     "cce_lse_forward": (
         _i32,
         [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64]
+        + [_i64] * 4 + [_i64] * 3 + [_f32, _i32, _ptr],
+    ),
+    "cce_lse_forward_static": (
+        _i32,
+        [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
         + [_i64] * 4 + [_i64] * 3 + [_f32, _i32, _ptr],
     ),
     "cce_indexed_neg_dot": (

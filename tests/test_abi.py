@@ -29,7 +29,7 @@ def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for want in ("cce_version", "cce_error_string", "cce_tile_stat_elems", "cce_lse_forward_workspace_bytes",
                  "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward",
-                 "cce_backward_dz"):
+                 "cce_backward_dz", "cce_lse_forward_static"):
         assert want in names
 
 
@@ -52,7 +52,7 @@ def test_host_only_queries():
     assert lib.cce_version() == _hip.ABI_VERSION
     assert lib.cce_error_string(0) == b"success"
     assert b"workspace" in lib.cce_error_string(10003)
-    # ceil(8192 / 32) * ceil(256000 / 128)
+    # ceil(8192 / 32) * ceil(256000 / 32)
     assert lib.cce_tile_stat_elems(8192, 256000) == 256 * 8000
     assert lib.cce_tile_stat_elems(33, 129) == 2 * 5
     assert lib.cce_tile_stat_elems(0, 100) == 0
@@ -72,3 +72,5 @@ def test_header_constants_match_binding():
     assert int(re.search(r"#define CCE_NUM_COUNTERS (\d+)", text).group(1)) == _hip.NUM_COUNTERS
     assert int(re.search(r"#define CCE_DTYPE_BF16 (\d+)", text).group(1)) == 0
     assert int(re.search(r"#define CCE_DTYPE_F16 (\d+)", text).group(1)) == 1
+    m = re.search(r"#define CCE_STATIC_SCRATCH_BYTES \((\d+) \* (\d+) \* (\d+)\)", text)
+    assert int(m.group(1)) * int(m.group(2)) * int(m.group(3)) == _hip.STATIC_SCRATCH_BYTES
