@@ -1,13 +1,14 @@
 """Benchmark of the linear-cross-entropy loss path on one MI355X.
 
-One step = forward + backward of ``linear_cross_entropy`` (impl="cce", gradient filtering on)
-over one batch of synthetic input already resident in HBM.  Workload: the Gemma-2-2B-shaped
-head, E [8192, 2304] bf16 ~ N(0,1), C [256000, 2304] bf16 ~ N(0, 0.02), uniform labels,
-softcap 30, reduction mean.  Prints one JSON line.
+One step = forward + backward of ``linear_cross_entropy`` over one batch of synthetic input already
+resident in HBM.  Default workload c2: the Gemma-2-2B-shaped head, E [8192, 2304] bf16 ~ N(0,1),
+C [256000, 2304] bf16 ~ N(0, 0.02), uniform labels, softcap 30, reduction mean, impl="cce" with gradient
+filtering.  ``--workload c1|c3|c4|c5|c5shard`` run the other benchmark configurations.  Prints one JSON line.
 
 The timing method restates the reference benchmark (benchmark/memory.py:82-112,
-benchmark/__main__.py:41-125): warm-up, then per iteration clear the gradients and run
-loss + backward between device-side time stamps.
+benchmark/__main__.py:41-125): warm-up, then per iteration clear the gradients and run loss + backward.
+The forward kernel and the backward are also timed one by one with device events recorded around their
+launches INSIDE the timed steps.
 """
 
 import argparse
@@ -22,32 +23,92 @@ for _p in (ROOT, os.path.join(ROOT, "ml-cross-entropy_amd")):
         sys.path.insert(0, _p)
 
 PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk x 2.4 GHz, dense
-# HBM bytes per launch of lse_forward_kernel at workload c2, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0
-# + WRITE_SIZE x 1.0, factors from a 1 GiB copy in the same runs; summary in profiles/).  A counter cannot be
-# read from inside this script, so the figure of the last profiled build is reported unless --traffic is given.
-MEASURED_TRAFFIC_BYTES = {"c2": 1.446e10}
+Z_LOSS_WEIGHT = 1e-4
+
+WORKLOADS = {
+    # name: N (rows of flattened e), D, V, and what the step does
+    "c1": dict(N=4096, D=1024, V=32000, softcap=None, impl="cce", text="5 % of the labels ignored, reduction=mean, impl=cce"),
+    "c2": dict(N=8192, D=2304, V=256000, softcap=30.0, impl="cce",
+               text="uniform labels, softcap=30.0, reduction=mean, impl=cce, gradient filter on"),
+    "c3": dict(N=16384, D=4096, V=128256, softcap=None, impl="cce",
+               text="E [4,4096,4096], labels [4,4096] with the last 256 per row ignored, shift=1, reduction=mean, impl=cce"),
+    "c4": dict(N=8192, D=2048, V=256000, softcap=None, impl="cce_kahan_full_c_full_e",
+               text="Zipf(1.1) labels, impl=cce_kahan_full_c_full_e (no filter), loss = nll + 1e-4 z-loss, reduction=none"),
+    "c5": dict(N=65536, D=3584, V=152064, softcap=None, impl="cce",
+               text="E = 4 C[label] + N(0,0.5) (peaked soft-max), reduction=mean, impl=cce, gradient filter on"),
+    "c5shard": dict(N=65536, D=3584, V=19008, softcap=None, impl="cce",
+                    text="the c5 inputs against the vocabulary shard C[0:19008] of 152064 classes, "
+                         "VocabParallelOptions(0, 19008), reduction=mean, impl=cce"),
+}
 
 
-def make_workload(name, device):
+def make_workload(name):
+    """Inputs on the CPU from one seeded generator in the fixed order E, C, labels (C first where E is
+    built from it), rounded to bf16."""
     import torch
 
+    spec = WORKLOADS[name]
+    N, D, V = spec["N"], spec["D"], spec["V"]
     g = torch.Generator().manual_seed(0)
-    if name == "c2":
-        N, D, V, softcap = 8192, 2304, 256000, 30.0
-    elif name == "c1":
-        N, D, V, softcap = 4096, 1024, 32000, None
+
+    def randn_bf16(rows, cols, std):
+        out = torch.empty((rows, cols), dtype=torch.bfloat16)
+        for s in range(0, rows, 16384):  # bounded host memory
+            n = min(16384, rows - s)
+            out[s : s + n] = (torch.randn((n, cols), generator=g) * std).to(torch.bfloat16)
+        return out
+
+    w = dict(spec, name=name, shift=0, vocab=V, vp=None)
+    if name in ("c5", "c5shard"):
+        Vfull = 152064
+        c = randn_bf16(Vfull, D, 0.02)
+        t = torch.randint(0, Vfull, (N,), generator=g)
+        e = torch.empty((N, D), dtype=torch.bfloat16)
+        for s in range(0, N, 8192):
+            idx = t[s : s + 8192]
+            e[s : s + 8192] = (4.0 * c[idx].float() + 0.5 * torch.randn((idx.numel(), D), generator=g)).to(torch.bfloat16)
+        if name == "c5shard":
+            c = c[:V].contiguous()
+            w["vp"] = (0, V)
+        w.update(e=e, c=c, t=t, valid=N)
+        return w
+    e = randn_bf16(N, D, 1.0)
+    c = randn_bf16(V, D, 0.02)
+    if name == "c4":  # Zipf(s = 1.1) over ranks 1..V by inverse-CDF sampling; rank r -> token r - 1
+        ranks = torch.arange(1, V + 1, dtype=torch.float64)
+        cdf = torch.cumsum(ranks.pow(-1.1), 0)
+        cdf /= cdf[-1].clone()
+        t = torch.searchsorted(cdf, torch.rand((N,), generator=g, dtype=torch.float64)).clamp_(max=V - 1)
     else:
-        raise ValueError(name)
-    e = torch.randn((N, D), generator=g).to(torch.bfloat16)
-    c = torch.empty((V, D), dtype=torch.bfloat16)
-    chunk = 32000
-    for s in range(0, V, chunk):  # bounded host memory
-        c[s : s + chunk] = (torch.randn((min(chunk, V - s), D), generator=g) * 0.02).to(torch.bfloat16)
-    t = torch.randint(0, V, (N,), generator=g)
+        t = torch.randint(0, V, (N,), generator=g)
+    valid = N
     if name == "c1":
-        idx = torch.randperm(N, generator=g)[: int(0.05 * N)]
-        t[idx] = -100
-    return dict(name=name, N=N, D=D, V=V, softcap=softcap, e=e, c=c, t=t)
+        t[torch.randperm(N, generator=g)[: int(0.05 * N)]] = -100
+        valid = int((t != -100).sum())
+    if name == "c3":
+        e, t = e.view(4, 4096, D), t.view(4, 4096)
+        t[:, -256:] = -100
+        w["shift"] = 1
+        valid = int((t[:, 1:] != -100).sum())
+    w.update(e=e, c=c, t=t, valid=valid)
+    return w
+
+
+def loss_fn(w):
+    """The step's forward as a closure over device tensors: returns a scalar loss."""
+    from cut_cross_entropy import VocabParallelOptions, linear_cross_entropy
+    from cut_cross_entropy.utils import compute_z_loss
+
+    vp = VocabParallelOptions(*w["vp"]) if w["vp"] is not None else None
+
+    def run(e, c, t):
+        if w["name"] == "c4":
+            nll, lse = linear_cross_entropy(e, c, t, reduction="none", return_lse=True, impl=w["impl"])
+            return (nll + Z_LOSS_WEIGHT * compute_z_loss(lse, t, reduction="none")).mean()
+        return linear_cross_entropy(e, c, t, softcap=w["softcap"], shift=w["shift"], reduction="mean", impl=w["impl"],
+                                    vocab_parallel_options=vp)
+
+    return run
 
 
 def cpu_baseline(w, rows):
@@ -59,9 +120,15 @@ def cpu_baseline(w, rows):
 
     threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     torch.set_num_threads(threads)
-    e = w["e"][:rows].float().requires_grad_(True)
+    e2 = w["e"].reshape(-1, w["D"])
+    t1 = w["t"].reshape(-1)
+    if w["shift"]:
+        e2, t1 = e2[: rows], t1[w["shift"] : rows + w["shift"]]
+    e = e2[:rows].float().requires_grad_(True)
     c = w["c"].float().requires_grad_(True)
-    t = w["t"][:rows]
+    t = t1[:rows].clone()
+    if w["vp"] is not None:
+        t[(t < w["vp"][0]) | (t >= w["vp"][1])] = -100  # out-of-shard targets contribute no correct-logit term
 
     def step():
         e.grad = c.grad = None
@@ -77,14 +144,14 @@ def cpu_baseline(w, rows):
         dt = time.perf_counter() - t0
         if dt > 12.0 or reps >= 5:
             break
-    valid = int((t != -100).sum())
+    valid = int((t != -100).sum()) if w["vp"] is None else rows
     return {
         "value": valid * reps / dt,
         "unit": "tokens/s",
         "cores": threads,
         "kind": "port",
         "sample": f"first {rows} of {w['N']} tokens against the full [{w['V']},{w['D']}] classifier, fp32, "
-                  f"dense oracle fwd+bwd, {reps} timed reps after 1 warm-up",
+                  f"dense oracle fwd+bwd (mean loss), {reps} timed reps after 1 warm-up",
     }
 
 
@@ -93,13 +160,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2")
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one plain 1 GiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--traffic", type=float, default=None,
-                    help="HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc (reported as given)")
+                    help="HBM bytes per launch of the dominant kernel of THIS build, measured with rocprofv3 --pmc; "
+                         "reported as given, null without it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives); use --gpus 1", file=sys.stderr)
@@ -110,24 +178,23 @@ def main():
     __graft_entry__.ensure_built()  # loads the library built in the tree; builds it only if there is none
     import torch
 
-    from cut_cross_entropy import _hip, linear_cross_entropy
+    from cut_cross_entropy import _hip
     from cut_cross_entropy import cce as cce_mod
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = make_workload(args.workload, dev)
+    w = make_workload(args.workload)
     e = w["e"].to(dev).requires_grad_(True)
     c = w["c"].to(dev).requires_grad_(True)
     t = w["t"].to(dev)
-    B = int((w["t"] != -100).sum())
-    N, V, D = w["N"], w["V"], w["D"]
-
+    B, N, V, D = w["valid"], w["N"], w["V"], w["D"]
+    run = loss_fn(w)
     counters = torch.zeros((4,), dtype=torch.int64, device=dev)
 
     def step():
         e.grad = None
         c.grad = None
-        loss = linear_cross_entropy(e, c, t, softcap=w["softcap"], reduction="mean", impl="cce")
+        loss = run(e, c, t)
         loss.backward()
         return loss
 
@@ -142,7 +209,9 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    # ---- timed region: exactly K steps -------------------------------------------------------
+    # ---- timed region: exactly K steps; device events around the kernels of every step ---------------
+    timers = {}
+    _hip.set_timers(timers)
     cce_mod.set_tile_counters(counters)
     counters.zero_()
     torch.cuda.synchronize()
@@ -152,9 +221,11 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     cce_mod.set_tile_counters(None)
+    _hip.set_timers(None)
     ms_per_step = dt / args.steps * 1e3
     cnt = [int(x) for x in counters.tolist()]
     k_r, k_e, k_c = (cnt[i] / max(cnt[0], 1) for i in (1, 2, 3))
+    kernel_ms = {name: sum(a.elapsed_time(b) for a, b in evs) / len(evs) for name, evs in timers.items()}
 
     # ---- loss-path peak memory (allocator peak minus the returned gradients) --------------------
     e.grad = c.grad = None
@@ -167,35 +238,12 @@ def main():
     grads = e.grad.numel() * e.grad.element_size() + c.grad.numel() * c.grad.element_size()
     extra_mb = (peak - grads) / 2**20
 
-    # ---- dominant kernel (fused matmul + LSE) timed alone with device events -----------------
-    lib = _hip.load()
-    ed, cd = e.detach(), c.detach()
-    lse = torch.empty((B,), dtype=torch.float32, device=dev)
-    tm = torch.empty((lib.cce_tile_stat_elems(B, V),), dtype=torch.float32, device=dev)
-    ws = torch.empty((lib.cce_lse_forward_workspace_bytes(B, V, D) // 8 + 1,), dtype=torch.int64, device=dev)
-    valids = None
-    if B != N:
-        valids = torch.nonzero(t != -100).squeeze(1).to(torch.int32)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def launch_fwd():
-        st = lib.cce_lse_forward(
-            ed.data_ptr(), cd.data_ptr(), None, valids.data_ptr() if valids is not None else None,
-            lse.data_ptr(), None, tm.data_ptr(), ws.data_ptr(), ws.numel() * 8,
-            N, B, V, D, ed.stride(0), cd.stride(0), cd.stride(1), w["softcap"] or 0.0, 0, stream)
-        assert st == 0
-
-    launch_fwd()
-    torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for a, b in evs:
-        a.record()
-        launch_fwd()
-        b.record()
-    torch.cuda.synchronize()
-    fwd_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    fwd_ms = kernel_ms["lse_forward"]
     fwd_flops = 2.0 * B * V * D
     fwd_tflops = fwd_flops / (fwd_ms * 1e-3) / 1e12
+    bwd_name = "backward_dense" if "backward_dense" in kernel_ms else "backward_sparse"
+    bwd_ms = kernel_ms[bwd_name]
+    bwd_flops = 2.0 * B * V * D * (k_r + k_e + k_c)
 
     f_alg = 2.0 * B * V * D * (1.0 + k_r + k_e + k_c)
     f_dense = 8.0 * B * V * D
@@ -213,8 +261,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{w['name']}: E[{N},{D}] bf16 N(0,1), C[{V},{D}] bf16 N(0,0.02), uniform labels, "
-                        f"softcap={w['softcap']}, reduction=mean, impl=cce, gradient filter on, fwd+bwd",
+            "workload": f"{w['name']}: E[{N},{D}] bf16, C[{V},{D}] bf16 N(0,0.02), {w['text']}, fwd+bwd",
             "valid_tokens": B,
         },
         "loss": float(loss),
@@ -224,14 +271,21 @@ def main():
         "fwd_bwd_frac_alg": f_alg / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "fwd_bwd_frac_dense_equiv": f_dense / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "roofline": {
-            "kernel": "lse_forward_kernel (fused E.C^T + softcap + online log-sum-exp)",
+            "kernel": "lse_forward_kernel (fused E.C^T + softcap + online log-sum-exp), device events around its "
+                      "launches inside the timed steps",
             "bound": "mfma",
             "achieved": fwd_tflops,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": fwd_tflops / PEAK_BF16_TFLOPS,
             "ms_per_launch": fwd_ms,
-            "traffic": args.traffic if args.traffic is not None else MEASURED_TRAFFIC_BYTES.get(w["name"]),
+            "traffic": args.traffic,
+        },
+        "backward": {
+            "path": bwd_name,
+            "ms": bwd_ms,
+            "tflops_alg": bwd_flops / (bwd_ms * 1e-3) / 1e12,
+            "frac_alg": bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         },
     }
     if not args.no_cpu_baseline:

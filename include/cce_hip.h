@@ -185,6 +185,41 @@ int cce_backward_dz(const void* e, const void* c, const void* bias,
                     float grad_scale, int64_t shift, int64_t target_offset,
                     float softcap, int dtype, void* stream);
 
+/* Workspace bytes of cce_backward_dense for a dz chunk buffer of at most `max_dz_bytes` (the function rounds
+ * it down to whole 256-class tiles of b rows and never goes below one tile), plus the fp32 dE accumulator
+ * [b, d] when `d_e_in_workspace` (d_e wanted in the 16-bit input type). */
+int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace,
+                                           int64_t max_dz_bytes);
+
+/*
+ * The whole unfiltered backward in one call: d_e, d_c, d_bias of cce_backward with the gradient filter
+ * off (filter_eps = None in cut_cross_entropy/cce_backward.py:346-521, i.e. the cce_exact / cce_kahan_full*
+ * presets).  Replaces the same Triton body (:20-310), both halves: the logit recompute and dz (:170-256) and
+ * the two products d_e += dz . c (:262-275), d_c += dz^T . e (:289-302), which the reference accumulates with
+ * atomics.  Here the vocabulary is walked in chunks; per chunk the dz of the chunk is written to the
+ * workspace in the input type, d_c[chunk] = dz^T . e and d_bias[chunk] = column sums of dz are complete and
+ * written once, and d_e accumulates over the chunks in fp32.
+ *
+ *   d_e      NULL or [n_rows, d]: float when d_e_is_fp32 (accumulated into: the caller zero-fills), else
+ *            `dtype` (rows of valid tokens are written once at the end; other rows are not touched)
+ *   d_c      NULL or [v, d] with the strides of c; float when d_c_is_fp32 else `dtype`; written, not accumulated
+ *   d_bias   NULL or [v] float, accumulated into
+ *   workspace  256-byte aligned; at least cce_backward_dense_workspace_bytes(b, v, d, d_e in `dtype`, 0) bytes.
+ *            Anything beyond that enlarges the chunks (fewer, better filled launches) up to 8192 classes.
+ * Layout requirements as for cce_backward_dz (16-byte aligned e, c and d_e, unit stride_cd, row strides that
+ * are multiples of 8, d a multiple of 64), else CCE_ERR_MISALIGNED and the caller uses cce_backward.
+ */
+int cce_backward_dense(const void* e, const void* c, const void* bias,
+                       const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                       const int32_t* valids, const int64_t* targets,
+                       void* d_e, void* d_c, float* d_bias,
+                       void* workspace, int64_t workspace_bytes,
+                       int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                       int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                       float grad_scale, int d_e_is_fp32, int d_c_is_fp32,
+                       int64_t shift, int64_t target_offset,
+                       float softcap, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,444 @@
+// cce_backward_dense: the unfiltered backward (gradient filter off) in one call.
+//
+// With every entry of dz = d loss / d logits in play the two gradient products are dense:
+//     dE[rows] = dz . C          dC = dz^T . E[rows]          dBias = column sums of dz
+// The reference forms them inside its one kernel with atomics on dE and dC
+// (cut_cross_entropy/cce_backward.py:258-310).  On this chip a tile of dz can feed register-resident
+// accumulators of only one of the two outputs at a time (a 256-row slab of dE or dC over D = 2304 .. 4096
+// columns is 2.4 .. 4 MB of fp32, against 0.5 MB of registers per compute unit) and global float atomics are
+// an order of magnitude too slow, so the vocabulary is walked in chunks and per chunk
+//   1. dense_dz_kernel    recomputes the logits of the chunk and writes dz [B, vc] in the input type
+//                         (the chunk is sized to stay in the last-level cache),
+//   2. dense_dc_kernel    dC[chunk] = dz^T . E : complete for these classes, written once,
+//   3. dense_de_kernel    dE += dz . C[chunk]  : accumulated in fp32 across the chunks (in d_e itself when the
+//                         caller asked for an fp32 dE, else in the workspace, converted at the end),
+//   4. dz_colsum_kernel   dBias[chunk], when wanted.
+// Both products run on the tile loop of cce_tile4.h (direct-to-LDS loads, LDS transpose reads for the
+// operand whose reduction index is the row index).  Everything is enqueued on the caller's stream; nothing
+// is allocated, no host synchronisation.
+#include <queue>
+#include <vector>
+
+#include "cce_dense.h"
+#include "cce_tile4.h"
+
+namespace cce {
+
+struct ProductParams {
+  const uint16_t* dz;   // [b][ldz]
+  int64_t ldz;
+  const uint16_t* c;    // first class of the chunk
+  int64_t stride_cv;
+  const uint16_t* e;
+  int64_t stride_e;
+  const int32_t* valids;
+  float* de_acc;        // fp32 accumulator of dE
+  int64_t ld_acc;
+  int acc_by_valids;    // rows of de_acc are rows of e (through valids) rather than valid-row numbers
+  void* d_c;            // first class of the chunk
+  int dc_fp32;
+  int64_t b;
+  int d;
+  int n_cls;            // classes in the chunk
+  int tiles_n;          // column tiles of either output
+  int dc_tiles, dc_per_xcd;  // tiles of dC (first in the grid: the longer reductions start first), per XCD slot count
+  int de_tiles, de_per_xcd;
+};
+
+constexpr int kProdThreads = 256;  // four waves, one per SIMD
+
+// Tile `block` of a group of `tiles` tiles: ids that land on one XCD get consecutive tiles, which share the A operand.
+__device__ __forceinline__ bool product_tile_of(int block, int tiles, int per_xcd, int tiles_n, int& tm, int& tn) {
+  const int xcd = block & 7;
+  const int slot = block >> 3;
+  const int lin = xcd * per_xcd + slot;
+  if (lin >= tiles) return false;
+  tm = lin / tiles_n;
+  tn = lin - tm * tiles_n;
+  return true;
+}
+
+// dE[row][col] += sum_class dz[row][class] * C[class][col]
+template <typename T>
+__device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, int tn, unsigned char* smem) {
+  using Tile = Tile4<T, false, true>;
+  typename Tile::Geometry g = Tile::geometry(smem);
+  const int64_t m0 = static_cast<int64_t>(tm) * Tile::TILE;
+  const int n0 = tn * Tile::TILE;
+
+  typename Tile::Source s;
+#pragma unroll
+  for (int q = 0; q < Tile::NQ1; ++q) {
+    int64_t i = m0 + Tile::row_direct(q, g.wave, g.lane);
+    i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
+    s.a_row[q] = p.dz + i * p.ldz + Tile::chunk_direct(g.wave, g.lane);
+  }
+  s.b_row[0] = nullptr;
+  s.a_km = nullptr;
+  s.a_stride = 0;
+  s.a_ok = true;
+  const int bcol = n0 + Tile::chunk_kmajor(g.wave, g.lane);
+  s.b_km = p.c + bcol;
+  s.b_ok = bcol < p.d;
+  s.b_stride = p.stride_cv;
+  s.b_rows = nullptr;
+  s.k_total = p.n_cls;
+  s.k_last = ((p.n_cls + Tile::BK - 1) / Tile::BK - 1) * Tile::BK;
+
+  f32x16 acc[Tile::WM][Tile::WN];
+  int ids[Tile::NQ1];
+  typename Tile::Ptrs ptrs;
+  Tile::prefetch(s, ptrs, ids, g);
+  Tile::run(acc, s, ptrs, ids, smem, g);
+
+#pragma unroll
+  for (int j = 0; j < Tile::WN; ++j) {
+    const int col = n0 + g.wn * 128 + j * 32 + g.l32;
+    if (col >= p.d) continue;
+#pragma unroll
+    for (int i = 0; i < Tile::WM; ++i) {
+      float* dst[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t row_i = m0 + g.wm * 128 + i * 32 + 8 * (r >> 2) + 4 * g.half + (r & 3);
+        dst[r] = nullptr;
+        if (row_i < p.b) {
+          const int64_t row = (p.acc_by_valids && p.valids != nullptr) ? static_cast<int64_t>(p.valids[row_i]) : row_i;
+          dst[r] = p.de_acc + row * p.ld_acc + col;
+        }
+      }
+      float old[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) old[r] = (dst[r] != nullptr) ? *dst[r] : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (dst[r] != nullptr) *dst[r] = old[r] + acc[i][j][r];
+    }
+  }
+}
+
+// dC[class][col] = sum_row dz[row][class] * E[row][col]
+template <typename T>
+__device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, int tn, unsigned char* smem) {
+  using Tile = Tile4<T, true, true>;
+  typename Tile::Geometry g = Tile::geometry(smem);
+  const int m0 = tm * Tile::TILE;
+  const int n0 = tn * Tile::TILE;
+
+  typename Tile::Source s;
+  s.a_row[0] = nullptr;
+  s.b_row[0] = nullptr;
+  const int chunk = Tile::chunk_kmajor(g.wave, g.lane);
+  s.a_km = p.dz + m0 + chunk;
+  s.a_ok = (m0 + chunk) < p.ldz;
+  s.a_stride = p.ldz;
+  s.b_km = p.e + n0 + chunk;
+  s.b_ok = (n0 + chunk) < p.d;
+  s.b_stride = p.stride_e;
+  s.b_rows = p.valids;
+  s.k_total = static_cast<int>(p.b);
+  s.k_last = 0;
+
+  f32x16 acc[Tile::WM][Tile::WN];
+  int ids[Tile::NQ1];
+  typename Tile::Ptrs ptrs;
+  Tile::prefetch(s, ptrs, ids, g);
+  Tile::run(acc, s, ptrs, ids, smem, g);
+
+#pragma unroll
+  for (int j = 0; j < Tile::WN; ++j) {
+    const int col = n0 + g.wn * 128 + j * 32 + g.l32;
+    if (col >= p.d) continue;
+#pragma unroll
+    for (int i = 0; i < Tile::WM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int cls = m0 + g.wm * 128 + i * 32 + 8 * (r >> 2) + 4 * g.half + (r & 3);
+        if (cls < p.n_cls) {
+          const int64_t off = static_cast<int64_t>(cls) * p.stride_cv + col;
+          if (p.dc_fp32) static_cast<float*>(p.d_c)[off] = acc[i][j][r];
+          else static_cast<uint16_t*>(p.d_c)[off] = Elem<T>::from_float(acc[i][j][r]);
+        }
+      }
+    }
+  }
+}
+
+// Both products of one chunk in one launch: the dC tiles (reduction over all B rows) take the first block ids,
+// the dE tiles (reduction over the classes of the chunk) the rest.  Blocks are handed to compute units in id
+// order as units fall free, so the two kinds fill each other's last round.
+template <typename T>
+__global__ __launch_bounds__(kProdThreads, 1) void dense_products_kernel(ProductParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int dc_blocks = p.dc_per_xcd * 8;
+  int tm, tn;
+  if (static_cast<int>(blockIdx.x) < dc_blocks) {
+    if (!product_tile_of(blockIdx.x, p.dc_tiles, p.dc_per_xcd, p.tiles_n, tm, tn)) return;
+    dense_dc_tile<T>(p, tm, tn, smem);
+  } else {
+    if (!product_tile_of(blockIdx.x - dc_blocks, p.de_tiles, p.de_per_xcd, p.tiles_n, tm, tn)) return;
+    dense_de_tile<T>(p, tm, tn, smem);
+  }
+}
+
+// dBias[class] = sum_row dz[row][class] over the chunk: 1024 threads = 16 row lanes x 64 classes.
+template <typename T>
+__global__ __launch_bounds__(1024) void dz_colsum_kernel(const uint16_t* dz, int64_t ldz, int64_t b, int n_cls, float* d_bias) {
+  __shared__ float part[16][64];
+  const int cl = threadIdx.x & 63;
+  const int rl = threadIdx.x >> 6;
+  const int cls = blockIdx.x * 64 + cl;
+  float sum = 0.0f;
+  if (cls < n_cls) {
+    for (int64_t i = rl; i < b; i += 16) sum += Elem<T>::to_float(dz[i * ldz + cls]);
+  }
+  part[rl][cl] = sum;
+  __syncthreads();
+  if (rl == 0 && cls < n_cls) {
+    float t = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) t += part[j][cl];  // fixed order: deterministic
+    d_bias[cls] += t;
+  }
+}
+
+__global__ void dense_fill_zero_kernel(float4* p, int64_t n4) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n4) p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+}
+
+// d_e[row of valid row i][:] = round(acc[i][:]), eight columns per thread
+template <typename T>
+__global__ void dense_store_de_kernel(const float* acc, const int32_t* valids, uint16_t* d_e, int64_t stride_e, int64_t b,
+                                      int d8) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= b * d8) return;
+  const int64_t i = idx / d8;
+  const int c8 = static_cast<int>(idx - i * d8);
+  const float4 lo = *reinterpret_cast<const float4*>(acc + (i * d8 + c8) * 8);
+  const float4 hi = *reinterpret_cast<const float4*>(acc + (i * d8 + c8) * 8 + 4);
+  uint4 out;
+  out.x = Elem<T>::pack2(lo.x, lo.y);
+  out.y = Elem<T>::pack2(lo.z, lo.w);
+  out.z = Elem<T>::pack2(hi.x, hi.y);
+  out.w = Elem<T>::pack2(hi.z, hi.w);
+  const int64_t row = valids ? static_cast<int64_t>(valids[i]) : i;
+  *reinterpret_cast<uint4*>(d_e + row * stride_e + c8 * 8) = out;
+}
+
+static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de,
+                                            bool want_dc);
+
+// Rounds the product launch of one chunk takes, in units of 256 reduction steps: n_long tiles of length
+// len_long and n_short tiles of len_short handed out in that order to 256 compute units as they fall free.
+static double product_makespan(int64_t n_long, int64_t len_long, int64_t n_short, int64_t len_short) {
+  const int cus = 256;
+  if (len_long < len_short) {
+    const int64_t n = n_long, l = len_long;
+    n_long = n_short; len_long = len_short; n_short = n; len_short = l;
+  }
+  // greedy list scheduling over a min-heap of the units' finishing times
+  std::priority_queue<int64_t, std::vector<int64_t>, std::greater<int64_t>> free_at;
+  for (int i = 0; i < cus; ++i) free_at.push(0);
+  int64_t worst = 0;
+  auto give = [&](int64_t n, int64_t len) {
+    for (int64_t t = 0; t < n; ++t) {
+      const int64_t end = free_at.top() + len;
+      free_at.pop();
+      free_at.push(end);
+      worst = end > worst ? end : worst;
+    }
+  };
+  give(n_long, len_long);
+  give(n_short, len_short);
+  return static_cast<double>(worst);
+}
+
+// Classes per chunk for a dz buffer of at most `max_dz_bytes`: a multiple of 256 up to 8192 that the buffer can
+// hold, chosen for the least estimated time per class: the dz kernel and the product launch (dC tiles with a
+// reduction over b rows, dE tiles with a reduction over vc classes, filling 256 compute units in rounds) plus a
+// fixed cost per launch that favours few, large chunks.  0: the buffer cannot hold 256 classes.
+static int64_t dense_chunk_classes(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de, bool want_dc) {
+  // the same question comes with every step of a training loop: remember the last answer of this thread
+  struct Memo {
+    int64_t b, v, d, bytes, answer;
+    bool de, dc;
+  };
+  static thread_local Memo memo = {0, 0, 0, 0, 0, false, false};
+  if (memo.b == b && memo.v == v && memo.d == d && memo.bytes == max_dz_bytes && memo.de == want_de && memo.dc == want_dc)
+    return memo.answer;
+  const int64_t answer = dense_chunk_classes_uncached(b, v, d, max_dz_bytes, want_de, want_dc);
+  memo = {b, v, d, max_dz_bytes, answer, want_de, want_dc};
+  return answer;
+}
+
+static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de,
+                                            bool want_dc) {
+  const int64_t v_pad = (v + 255) / 256 * 256;
+  int64_t top = max_dz_bytes / (b * 2) / 256 * 256;
+  if (top > 8192) top = 8192;
+  if (top < 256) return 0;
+  if (top >= v_pad) return v_pad;
+  const int64_t col_tiles = (d + 255) / 256;
+  const int64_t row_tiles = (b + 255) / 256;
+  int64_t best = top;
+  double best_cost = 1e300;
+  for (int64_t vc = top; vc >= 256; vc -= 256) {
+    const int64_t chunks = (v + vc - 1) / vc;
+    const double products = product_makespan(want_dc ? vc / 256 * col_tiles : 0, (b + 255) / 256,
+                                             want_de ? row_tiles * col_tiles : 0, vc / 256);
+    // dz: row_tiles x (vc / 256) logit tiles of d / 256 units each, in rounds of 256 as well
+    const int64_t dz_tiles = row_tiles * (vc / 256);
+    const double dz = static_cast<double>((dz_tiles + 255) / 256) * static_cast<double>(col_tiles);
+    // One unit (256 reduction steps of a tile) is about 3.9 us.  Per chunk: two launches with their gaps, fill and
+    // drain (~ 10 us each), and the read-modify-write of the fp32 dE accumulator (b x d x 8 bytes at ~ 3.5 TB/s),
+    // which all tiles of a round do at the same time.
+    const double per_launch = 2.5;
+    const double rmw = want_de ? static_cast<double>(b) * static_cast<double>(d) * 8.0 / 3.5e12 / 3.9e-6 : 0.0;
+    const double cost = static_cast<double>(chunks) * (products + dz + 2.0 * per_launch + rmw);
+    if (cost < best_cost * (1.0 - 1e-9)) {
+      best = vc;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+static int64_t align256(int64_t x) { return (x + 255) / 256 * 256; }
+
+}  // namespace cce
+
+using namespace cce;
+
+extern "C" int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace,
+                                                      int64_t max_dz_bytes) {
+  if (b <= 0 || v <= 0 || d <= 0) return 0;
+  int64_t vc = dense_chunk_classes(b, v, d, max_dz_bytes, true, true);
+  if (vc == 0) vc = 256;  // the smallest plan
+  const int64_t acc = d_e_in_workspace ? align256(b * d * 4) : 0;
+  return acc + align256(b * vc * 2);
+}
+
+extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias,
+                                  const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                                  const int32_t* valids, const int64_t* targets,
+                                  void* d_e, void* d_c, float* d_bias,
+                                  void* workspace, int64_t workspace_bytes,
+                                  int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                                  int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                                  float grad_scale, int d_e_is_fp32, int d_c_is_fp32,
+                                  int64_t shift, int64_t target_offset,
+                                  float softcap, int dtype, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (b < 0 || v <= 0 || d <= 0 || n_rows < 0 || shift < 0) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0) return CCE_OK;
+  if (e == nullptr || c == nullptr || lse == nullptr || d_out == nullptr || targets == nullptr)
+    return CCE_ERR_INVALID_ARGUMENT;
+  if (valids == nullptr && b > n_rows) return CCE_ERR_INVALID_ARGUMENT;
+  if (n_rows >= (int64_t(1) << 31) || b >= (int64_t(1) << 31) - 512 || v >= (int64_t(1) << 31) - 512 || d > (1 << 24))
+    return CCE_ERR_INVALID_ARGUMENT;
+  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+  if (d_e == nullptr && d_c == nullptr && d_bias == nullptr) return CCE_OK;
+  if (!aligned16(e) || !aligned16(c) || d % kDmaBK != 0 || stride_e % 8 != 0 || stride_cv % 8 != 0 || stride_cd != 1)
+    return CCE_ERR_MISALIGNED;
+  if (stride_e >= (int64_t(1) << 30) || stride_cv >= (int64_t(1) << 30)) return CCE_ERR_INVALID_ARGUMENT;
+  if (d_e != nullptr && !aligned16(d_e)) return CCE_ERR_MISALIGNED;
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+    return workspace == nullptr ? CCE_ERR_WORKSPACE_TOO_SMALL : CCE_ERR_MISALIGNED;
+
+  // ---- plan: [fp32 dE accumulator][dz chunk] -------------------------------------------------------------
+  const bool acc_in_ws = (d_e != nullptr) && !d_e_is_fp32;
+  const int64_t acc_bytes = acc_in_ws ? align256(b * d * 4) : 0;
+  // the plan the size query made (both gradients wanted), so that its answer always suffices
+  const int64_t vc = dense_chunk_classes(b, v, d, workspace_bytes - acc_bytes, true, true);
+  if (vc == 0) return CCE_ERR_WORKSPACE_TOO_SMALL;
+  float* acc = acc_in_ws ? static_cast<float*>(workspace) : static_cast<float*>(d_e);
+  uint16_t* dz = reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + acc_bytes);
+  const int64_t ldz = vc;
+
+  if (acc_in_ws) {
+    const int64_t n4 = b * d / 4;
+    hipLaunchKernelGGL(dense_fill_zero_kernel, dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<float4*>(acc), n4);
+  }
+
+  ProductParams p;
+  p.dz = dz;
+  p.ldz = ldz;
+  p.stride_cv = stride_cv;
+  p.e = static_cast<const uint16_t*>(e);
+  p.stride_e = stride_e;
+  p.valids = valids;
+  p.de_acc = acc;
+  p.ld_acc = acc_in_ws ? d : stride_e;
+  p.acc_by_valids = acc_in_ws ? 0 : 1;
+  p.dc_fp32 = d_c_is_fp32;
+  p.b = b;
+  p.d = static_cast<int>(d);
+
+  using TileB = Tile4<BF16, true, true>;
+  const int lds = TileB::LDS_BYTES;
+  const int tiles_n = static_cast<int>((d + 255) / 256);
+  hipError_t err;
+#define CCE_LAUNCH_PRODUCT(KERN, BLOCKS)                                                            \
+  do {                                                                                              \
+    auto kern = KERN;                                                                               \
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                  \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                     \
+    if (err != hipSuccess) return status_from_hip(err);                                             \
+    hipLaunchKernelGGL(kern, dim3(BLOCKS), dim3(kProdThreads), lds, stream, p);                     \
+  } while (0)
+
+  const size_t es = 2;
+  for (int64_t v0 = 0; v0 < v; v0 += vc) {
+    const int64_t n = (v - v0 < vc) ? (v - v0) : vc;
+    const unsigned char* c_chunk = static_cast<const unsigned char*>(c) + v0 * stride_cv * es;
+    const void* bias_chunk = bias ? static_cast<const unsigned char*>(bias) + v0 * es : nullptr;
+    int st = dense_dz_launch(e, c_chunk, bias_chunk, lse, d_out, d_out_is_scalar, d_lse, valids, targets, dz, ldz, 0, 1,
+                             n_rows, b, n, d, stride_e, stride_cv, stride_cd, grad_scale, shift, target_offset + v0,
+                             softcap, dtype, stream);
+    if (st != CCE_OK) return st;
+    p.c = reinterpret_cast<const uint16_t*>(c_chunk);
+    p.n_cls = static_cast<int>(n);
+    p.tiles_n = tiles_n;
+    p.d_c = nullptr;
+    p.dc_tiles = 0;
+    if (d_c != nullptr) {
+      p.d_c = static_cast<unsigned char*>(d_c) + v0 * stride_cv * (d_c_is_fp32 ? 4 : 2);
+      p.dc_tiles = static_cast<int>((n + 255) / 256) * tiles_n;
+    }
+    p.dc_per_xcd = (p.dc_tiles + 7) / 8;
+    p.de_tiles = (d_e != nullptr) ? static_cast<int>((b + 255) / 256) * tiles_n : 0;
+    p.de_per_xcd = (p.de_tiles + 7) / 8;
+    const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
+    if (blocks > 0) {
+      if (dtype == CCE_DTYPE_BF16) CCE_LAUNCH_PRODUCT(dense_products_kernel<BF16>, blocks);
+      else CCE_LAUNCH_PRODUCT(dense_products_kernel<F16>, blocks);
+    }
+    if (d_bias != nullptr) {
+      const unsigned blocks = static_cast<unsigned>((n + 63) / 64);
+      if (dtype == CCE_DTYPE_BF16)
+        hipLaunchKernelGGL(dz_colsum_kernel<BF16>, dim3(blocks), dim3(1024), 0, stream, dz, ldz, b, static_cast<int>(n),
+                           d_bias + v0);
+      else
+        hipLaunchKernelGGL(dz_colsum_kernel<F16>, dim3(blocks), dim3(1024), 0, stream, dz, ldz, b, static_cast<int>(n),
+                           d_bias + v0);
+    }
+    err = hipGetLastError();
+    if (err != hipSuccess) return status_from_hip(err);
+  }
+#undef CCE_LAUNCH_PRODUCT
+
+  if (acc_in_ws) {
+    const int d8 = static_cast<int>(d / 8);
+    const int64_t total = b * d8;
+    const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+    if (dtype == CCE_DTYPE_BF16)
+      hipLaunchKernelGGL(dense_store_de_kernel<BF16>, dim3(blocks), dim3(256), 0, stream, acc, valids,
+                         static_cast<uint16_t*>(d_e), stride_e, b, d8);
+    else
+      hipLaunchKernelGGL(dense_store_de_kernel<F16>, dim3(blocks), dim3(256), 0, stream, acc, valids,
+                         static_cast<uint16_t*>(d_e), stride_e, b, d8);
+  }
+  return status_from_hip(hipGetLastError());
+}

@@ -5,7 +5,7 @@
 // them as such on the chunk.  The kernel is the forward kernel with another epilogue: same work
 // items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as whole rows
 // of 256 bytes per wave instruction after a transposition through LDS.
-#include "cce_common.h"
+#include "cce_dense.h"
 
 namespace cce {
 
@@ -25,6 +25,8 @@ struct DzParams {
   int64_t shift, target_offset;
   float grad_scale;
   int d_out_is_scalar;
+  int pad_store;  // also store the (zero) gradients of the classes between v and the end of their 16-byte piece,
+                  // up to column ldz: the product kernels read dz in whole 64-class stages
   int nrb, nvt, nsplit, nitems, items_per_xcd;
   Softcap sc;
 };
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
           const int64_t gcol = static_cast<int64_t>(cls0) + vh * (32 * kViPer) + pc * kPieceElems;
           if (gi < p.b) {
             unsigned char* dst = static_cast<unsigned char*>(p.dz) + (gi * p.ldz + gcol) * kEs;
-            if (!GENERAL || gcol + kPieceElems <= p.v) {
+            if (!GENERAL || gcol + kPieceElems <= p.v || (p.pad_store && gcol + kPieceElems <= p.ldz)) {
               *reinterpret_cast<uint4*>(dst) = val;
             } else if (OUT32) {
               const uint32_t w[4] = {val.x, val.y, val.z, val.w};
@@ -208,19 +210,14 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
   }
 }
 
-}  // namespace cce
-
-using namespace cce;
-
-extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
-                               const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
-                               const int32_t* valids, const int64_t* targets,
-                               void* dz, int64_t ldz, int dz_is_fp32,
-                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
-                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
-                               float grad_scale, int64_t shift, int64_t target_offset,
-                               float softcap, int dtype, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+int dense_dz_launch(const void* e, const void* c, const void* bias,
+                    const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                    const int32_t* valids, const int64_t* targets,
+                    void* dz, int64_t ldz, int dz_is_fp32, int pad_store,
+                    int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                    int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                    float grad_scale, int64_t shift, int64_t target_offset,
+                    float softcap, int dtype, hipStream_t stream) {
   if (b < 0 || v <= 0 || d <= 0 || n_rows < 0 || shift < 0 || ldz < v) return CCE_ERR_INVALID_ARGUMENT;
   if (b == 0) return CCE_OK;
   if (e == nullptr || c == nullptr || lse == nullptr || d_out == nullptr || targets == nullptr || dz == nullptr)
@@ -254,6 +251,7 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
   p.target_offset = target_offset;
   p.grad_scale = grad_scale;
   p.d_out_is_scalar = d_out_is_scalar;
+  p.pad_store = pad_store;
   p.nrb = static_cast<int>((b + kDzTile - 1) / kDzTile);
   p.nvt = static_cast<int>((v + kDzTile - 1) / kDzTile);
   p.nsplit = choose_span_count(p.nrb, p.nvt);
@@ -286,4 +284,19 @@ extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
 #undef CCE_LAUNCH_DZ
 #undef CCE_LAUNCH_DZ2
   return status_from_hip(hipGetLastError());
+}
+
+}  // namespace cce
+
+extern "C" int cce_backward_dz(const void* e, const void* c, const void* bias,
+                               const float* lse, const float* d_out, int d_out_is_scalar, const float* d_lse,
+                               const int32_t* valids, const int64_t* targets,
+                               void* dz, int64_t ldz, int dz_is_fp32,
+                               int64_t n_rows, int64_t b, int64_t v, int64_t d,
+                               int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
+                               float grad_scale, int64_t shift, int64_t target_offset,
+                               float softcap, int dtype, void* stream) {
+  return cce::dense_dz_launch(e, c, bias, lse, d_out, d_out_is_scalar, d_lse, valids, targets, dz, ldz, dz_is_fp32, 0,
+                              n_rows, b, v, d, stride_e, stride_cv, stride_cd, grad_scale, shift, target_offset, softcap,
+                              dtype, static_cast<hipStream_t>(stream));
 }

@@ -1,0 +1,366 @@
+// One 256 x 256 tile of  Out[m][n] = sum_k A[m][k] * B[k][n]  on one compute unit with FOUR waves, one per
+// SIMD, each owning 128 x 128 of the tile: 4 x 4 accumulator blocks of 32 x 32 = 256 accumulation registers.
+// Per 16 reduction steps a wave reads 4 + 4 operand fragments for 16 MFMAs -- two thirds of the LDS reads per
+// MFMA of a 2 x 4 arrangement of eight waves (6 for 8).  LDS instruction issue, shared between these reads and
+// the incoming direct-to-LDS loads, is what bounds these kernels next to the matrix pipeline itself.  With one
+// wave per SIMD nothing else hides a wave's own instruction issue, so the main loop is kept lean: every LDS
+// address is a per-lane base plus an immediate, load pointers are formed one per MFMA slot a step ahead.
+//
+// Either operand is streamed through LDS by direct global -> LDS loads (`global_load_lds_dwordx4`), in one
+// of two layouts:
+//   Direct   the operand's rows are tile rows (m or n) and the reduction index is contiguous in memory:
+//            LDS image 256 rows x 128 bytes (64 k), 16-byte chunks XOR-swizzled with (row >> 1) & 7; one load
+//            instruction fills 8 rows; a fragment is one 16-byte read.
+//   KMajor   the matrix is [K][256] row-major (reduction index = row): LDS image 64 rows x 512 bytes, the 32
+//            chunks of a row XOR-swizzled with 4 (row & 3); one load instruction fills 2 rows; a fragment is
+//            two LDS transpose reads (`ds_read_b64_tr_b16`) of four k rows each.  In one such read a group
+//            of 16 lanes supplies 16 addresses of 4 elements -- lane i: row r0 + (i >> 2), columns
+//            c0 + 4 (i & 3) .. + 3 -- and lane i receives the elements [r0 .. r0 + 3][c0 + i].
+// A row of a KMajor operand that does not exist (k past the end of the reduction, a column chunk past the
+// matrix) is fetched from a line of zeros, so a non-finite value elsewhere never meets the product.
+//
+// A stage is 64 reduction steps (32 KB per operand), two stages in LDS, one barrier per stage.  The loads of a
+// stage are issued in two groups of 8, one load after every second MFMA: A under the last 16-step of the
+// stage before last, B under the first 16-step of the stage before; the fragment reads of step k + 1 go out
+// between the MFMAs of step k.  Completion of the loads is tracked by hand (s_waitcnt vmcnt), the compiler
+// cannot see them.
+#pragma once
+
+#include "cce_common.h"
+
+namespace cce {
+
+static __device__ __align__(256) uint16_t g_zero_line[128];  // never written
+
+typedef short tr_short4_t __attribute__((ext_vector_type(4)));
+
+template <typename T, bool A_KM, bool B_KM>
+struct Tile4 {
+  static constexpr int WM = 4, WN = 4;   // accumulator blocks per wave
+  static constexpr int NW = 4;           // waves, 2 (m) x 2 (n)
+  static constexpr int NT = 64 * NW;
+  static constexpr int TILE = 256;
+  static constexpr int BK = 64;
+  static constexpr int OP_BYTES = 32 * 1024;
+  static constexpr int STAGE_BYTES = 2 * OP_BYTES;
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int NQ1 = 8;          // loads per wave, stage and operand
+  using vec8 = typename Elem<T>::vec8;
+
+  // ---- what a lane fetches ---------------------------------------------------------------------------
+  static __device__ __forceinline__ int row_direct(int q, int wave, int lane) { return 8 * (q * NW + wave) + (lane >> 3); }
+  static __device__ __forceinline__ int chunk_direct(int wave, int lane) {
+    const int sw = (4 * (wave & 1) + (lane >> 4)) & 7;  // (row >> 1) & 7
+    return ((lane & 7) ^ sw) * 8;
+  }
+  // KMajor: load q of a wave covers stage rows 8 q + 2 wave + (lane >> 5)
+  static __device__ __forceinline__ int row_kmajor(int q, int wave, int lane) { return 2 * (q * NW + wave) + (lane >> 5); }
+  static __device__ __forceinline__ int chunk_kmajor(int wave, int lane) {
+    const int r3 = (2 * (wave & 1) + (lane >> 5)) & 3;  // row & 3
+    return ((lane & 31) ^ (r3 << 2)) * 8;
+  }
+
+  struct Source {
+    const uint16_t* a_row[A_KM ? 1 : NQ1];  // Direct: row base + chunk_direct, one row per load
+    const uint16_t* b_row[B_KM ? 1 : NQ1];
+    const uint16_t* a_km;   // KMajor: matrix base + first column of the tile + chunk_kmajor
+    const uint16_t* b_km;
+    int64_t a_stride;       // KMajor: elements between consecutive k rows (< 2^30)
+    int64_t b_stride;
+    const int32_t* b_rows;  // KMajor B: optional gather of its k rows (nullptr: rows 0 .. K - 1)
+    bool a_ok;              // KMajor: this lane's chunk lies inside the matrix
+    bool b_ok;
+    int k_total;            // length of the reduction
+    int k_last;             // first reduction index of the last stage (a Direct operand never reads past it)
+  };
+
+  // Per-lane constants of the main loop.
+  struct Geometry {
+    int lane, wave, wm, wn, l32, half;
+    unsigned lds_base;
+    // LDS byte addresses (inside a stage) of this lane's fragment reads
+    int a_addr[4];  // Direct: one per 16-step kk (block i adds i * 4096); KMajor: one per block i (kk adds kk * 8192)
+    int b_addr[4];
+  };
+  static __device__ __forceinline__ Geometry geometry(unsigned char* lds) {
+    Geometry g;
+    g.lane = threadIdx.x & 63;
+    g.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    g.wm = g.wave >> 1;
+    g.wn = g.wave & 1;
+    g.l32 = g.lane & 31;
+    g.half = g.lane >> 5;
+    g.lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+    const int sw = (g.l32 >> 1) & 7;
+    const int tr_row = 8 * (g.lane >> 5) + ((g.lane >> 2) & 3);
+    const int tr_col = 16 * ((g.lane >> 4) & 1) + 4 * (g.lane & 3);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      if (A_KM) {
+        const int col = g.wm * 128 + x * 32 + tr_col;
+        g.a_addr[x] = tr_row * 512 + ((((col >> 3) ^ ((tr_row & 3) << 2)) << 4) | ((col & 7) << 1));
+      } else {
+        g.a_addr[x] = (g.wm * 128 + g.l32) * 128 + (((x * 2 + g.half) ^ sw) << 4);
+      }
+      if (B_KM) {
+        const int col = g.wn * 128 + x * 32 + tr_col;
+        g.b_addr[x] = OP_BYTES + tr_row * 512 + ((((col >> 3) ^ ((tr_row & 3) << 2)) << 4) | ((col & 7) << 1));
+      } else {
+        g.b_addr[x] = OP_BYTES + (g.wn * 128 + g.l32) * 128 + (((x * 2 + g.half) ^ sw) << 4);
+      }
+    }
+    return g;
+  }
+
+  // Sources of the loads of one stage for the KMajor operands, formed a step ahead of their use (a Direct
+  // operand's pointer is its row pointer plus a scalar, formed when the load is issued).
+  struct Ptrs {
+    const uint16_t* a[A_KM ? NQ1 : 1];
+    const uint16_t* b[B_KM ? NQ1 : 1];
+  };
+
+  static __device__ __forceinline__ const uint16_t* zero_line(const Geometry& g) { return g_zero_line + (g.lane & 15) * 8; }
+
+  // Pointer of load q of operand A for the stage that starts at k0.
+  static __device__ __forceinline__ void prep_a(Ptrs& p, int q, const Source& s, int k0, const Geometry& g) {
+    if (A_KM) {
+      const int row = k0 + row_kmajor(q, g.wave, g.lane);
+      const uint16_t* ptr = s.a_km + static_cast<uint64_t>(static_cast<uint32_t>(row)) * static_cast<uint32_t>(s.a_stride);
+      p.a[A_KM ? q : 0] = (s.a_ok && row < s.k_total) ? ptr : zero_line(g);
+    }
+  }
+  // Row of a gathered KMajor B for load q of the stage that starts at k0 (-1: none).
+  static __device__ __forceinline__ void prep_b_id(int (&ids)[NQ1], int q, const Source& s, int k0, const Geometry& g) {
+    if (!B_KM) return;
+    const int row = k0 + row_kmajor(q, g.wave, g.lane);
+    int id = -1;
+    if (row < s.k_total) id = (s.b_rows != nullptr) ? s.b_rows[row] : row;
+    ids[q] = id;
+  }
+  static __device__ __forceinline__ void prep_b(Ptrs& p, int q, const int (&ids)[NQ1], const Source& s, int k0,
+                                                const Geometry& g) {
+    if (B_KM) {
+      const uint16_t* ptr = s.b_km + static_cast<uint64_t>(static_cast<uint32_t>(ids[q])) * static_cast<uint32_t>(s.b_stride);
+      p.b[B_KM ? q : 0] = (s.b_ok && ids[q] >= 0) ? ptr : zero_line(g);
+    }
+  }
+
+  // Load q of the stage that starts at k0 into LDS stage STAGE (a Direct operand past the end of the reduction
+  // fetches its last stage again: never consumed).
+  template <int STAGE>
+  static __device__ __forceinline__ void issue_a(const Ptrs& p, int q, const Source& s, int k0, const Geometry& g) {
+    const uint16_t* src = A_KM ? p.a[A_KM ? q : 0] : s.a_row[A_KM ? 0 : q] + min(k0, s.k_last);
+    lds_dma16(src, g.lds_base + STAGE * STAGE_BYTES + (q * NW + g.wave) * 1024);
+  }
+  template <int STAGE>
+  static __device__ __forceinline__ void issue_b(const Ptrs& p, int q, const Source& s, int k0, const Geometry& g) {
+    const uint16_t* src = B_KM ? p.b[B_KM ? q : 0] : s.b_row[B_KM ? 0 : q] + min(k0, s.k_last);
+    lds_dma16(src, g.lds_base + STAGE * STAGE_BYTES + OP_BYTES + (q * NW + g.wave) * 1024);
+  }
+
+  // ---- fragment reads --------------------------------------------------------------------------------
+  struct Frags {
+    vec8 a[WM];
+    vec8 b[WN];
+  };
+  struct Half {
+    tr_short4_t lo, hi;
+  };
+  static __device__ __forceinline__ tr_short4_t read_tr(const unsigned char* lds, int addr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tr_short4_t*)(lds + addr));
+  }
+  static __device__ __forceinline__ vec8 read_16(const unsigned char* lds, int addr) {
+    return __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(lds + addr));
+  }
+  static constexpr int kReadsA = A_KM ? 2 : 1;
+  static constexpr int kReadsB = B_KM ? 2 : 1;
+  static constexpr int kReads = WM * kReadsA + WN * kReadsB;
+  // part `part` of the read of fragment a[i] / b[i] of step KK of stage STAGE: the address is a lane constant
+  // plus a compile-time offset.
+  template <int STAGE, int KK>
+  static __device__ __forceinline__ void read_a(int i, int part, Frags& f, Half (&h)[WM], const unsigned char* lds,
+                                                const Geometry& g) {
+    if (A_KM) {
+      const tr_short4_t v = read_tr(lds, g.a_addr[i] + STAGE * STAGE_BYTES + KK * 16 * 512 + part * 4 * 512);
+      if (part) h[i].hi = v; else h[i].lo = v;
+      if (part) f.a[i] = __builtin_bit_cast(vec8, h[i]);
+    } else {
+      f.a[i] = read_16(lds, g.a_addr[KK] + STAGE * STAGE_BYTES + i * 32 * 128);
+    }
+  }
+  template <int STAGE, int KK>
+  static __device__ __forceinline__ void read_b(int i, int part, Frags& f, Half (&h)[WN], const unsigned char* lds,
+                                                const Geometry& g) {
+    if (B_KM) {
+      const tr_short4_t v = read_tr(lds, g.b_addr[i] + STAGE * STAGE_BYTES + KK * 16 * 512 + part * 4 * 512);
+      if (part) h[i].hi = v; else h[i].lo = v;
+      if (part) f.b[i] = __builtin_bit_cast(vec8, h[i]);
+    } else {
+      f.b[i] = read_16(lds, g.b_addr[KK] + STAGE * STAGE_BYTES + i * 32 * 128);
+    }
+  }
+  // Read op r of a step, in the order the MFMAs (m-major) want their operands: a0, b0 .. b3, a1, a2, a3.
+  template <int STAGE, int KK>
+  static __device__ __forceinline__ void read_op(int r, Frags& f, Half (&ha)[WM], Half (&hb)[WN], const unsigned char* lds,
+                                                 const Geometry& g) {
+    if (r < kReadsA) {
+      read_a<STAGE, KK>(0, r, f, ha, lds, g);
+    } else if (r < kReadsA + WN * kReadsB) {
+      const int j = r - kReadsA;
+      read_b<STAGE, KK>(j / kReadsB, j % kReadsB, f, hb, lds, g);
+    } else {
+      const int j = r - kReadsA - WN * kReadsB;
+      read_a<STAGE, KK>(1 + j / kReadsA, j % kReadsA, f, ha, lds, g);
+    }
+  }
+  template <int STAGE, int KK>
+  static __device__ __forceinline__ void read_all(Frags& f, const unsigned char* lds, const Geometry& g) {
+    Half ha[WM], hb[WN];
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) read_op<STAGE, KK>(r, f, ha, hb, lds, g);
+  }
+
+  // What a 16-step does between its MFMAs besides the fragment reads of the next step:
+  //   kIssueB  + loads of B for the stage at kl into LDS stage LSTAGE, one after every odd MFMA
+  //   kPrepIds + row lookups of a gathered B for the stage at k0, one after every even MFMA
+  //   kPrepA   + pointers of the A loads for the stage at k0
+  //   kIssueAPrepB  loads of A for the stage at kl into LDS stage LSTAGE after the odd MFMAs, pointers of the B
+  //                 loads (from `ids`) for the stage at k0 after the even ones
+  enum Extra { kNone, kIssueB, kPrepIds, kPrepA, kIssueAPrepB };
+
+  // The 16 MFMAs on `cur`; between them the reads of fragment set `nxt` (step RKK of stage RSTAGE) and EXTRA.
+  template <int RSTAGE, int RKK, Extra EXTRA, int LSTAGE>
+  static __device__ __forceinline__ void step(f32x16 (&acc)[WM][WN], const Frags& cur, Frags& nxt, const unsigned char* lds,
+                                              const Source& s, int kl, int k0, Ptrs& ptrs, int (&ids)[NQ1],
+                                              const Geometry& g) {
+    constexpr int kMfmas = WM * WN;
+    Half ha[WM], hb[WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        acc[i][j] = Elem<T>::mfma(cur.a[i], cur.b[j], acc[i][j]);
+        const int idx = i * WN + j;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = idx * kReads / kMfmas; r < (idx + 1) * kReads / kMfmas; ++r)
+          read_op<RSTAGE, RKK>(r, nxt, ha, hb, lds, g);
+        const int q = idx >> 1;
+        if (idx & 1) {
+          if (EXTRA == kIssueB) issue_b<LSTAGE>(ptrs, q, s, kl, g);
+          if (EXTRA == kIssueAPrepB) issue_a<LSTAGE>(ptrs, q, s, kl, g);
+        } else {
+          if (EXTRA == kPrepIds) prep_b_id(ids, q, s, k0, g);
+          if (EXTRA == kPrepA) prep_a(ptrs, q, s, k0, g);
+          if (EXTRA == kIssueAPrepB) prep_b(ptrs, q, ids, s, k0, g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  }
+
+  // Start fetching a tile into the idle LDS ring: all of stage 0 and the A loads of stage 1; leaves in `ptrs.b`
+  // the B pointers of stage 1.  A caller with work between two tiles (an epilogue) calls this first, so that
+  // the next main loop starts with data in LDS.
+  static __device__ __forceinline__ void prefetch(const Source& s, Ptrs& ptrs, int (&ids)[NQ1], const Geometry& g) {
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) {
+      prep_a(ptrs, q, s, 0, g);
+      prep_b_id(ids, q, s, 0, g);
+    }
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) prep_b(ptrs, q, ids, s, 0, g);
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) issue_a<0>(ptrs, q, s, 0, g);
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) issue_b<0>(ptrs, q, s, 0, g);
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) {
+      prep_a(ptrs, q, s, BK, g);
+      prep_b_id(ids, q, s, BK, g);
+    }
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) issue_a<1>(ptrs, q, s, BK, g);
+#pragma unroll
+    for (int q = 0; q < NQ1; ++q) prep_b(ptrs, q, ids, s, BK, g);
+  }
+
+  // One stage (four 16-steps) whose data sits in LDS stage CUR; `fa` holds its first fragment set on entry and
+  // that of the next stage on exit.
+  template <int CUR>
+  static __device__ __forceinline__ void stage(f32x16 (&acc)[WM][WN], Frags& fa, Frags& fb, const unsigned char* lds,
+                                               const Source& s, int st, Ptrs& ptrs, int (&ids)[NQ1], const Geometry& g) {
+    constexpr int NXT = 1 - CUR;
+    const int k1 = (st + 1) * BK;
+    const int k2 = (st + 2) * BK;
+    step<CUR, 1, kIssueB, NXT>(acc, fa, fb, lds, s, k1, k2, ptrs, ids, g);    // the B loads of stage st + 1
+    step<CUR, 2, kPrepIds, NXT>(acc, fb, fa, lds, s, k1, k2, ptrs, ids, g);   // rows of B for stage st + 2
+    step<CUR, 3, kPrepA, NXT>(acc, fa, fb, lds, s, k1, k2, ptrs, ids, g);     // pointers of A for stage st + 2
+    // Stage st + 1 has landed for this wave; after the barrier for every wave, and every wave holds its last
+    // fragments of stage st in registers: that LDS stage is free for stage st + 2.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (B_KM) {
+      // The looked-up rows are pinned as used here, where nothing is in flight: the compiler places its own
+      // wait for them at their first use, and further down it would also wait for the direct-to-LDS loads.
+#pragma unroll
+      for (int q = 0; q < NQ1; ++q) asm volatile("" : "+v"(ids[q]));
+    }
+    __syncthreads();
+    step<NXT, 0, kIssueAPrepB, CUR>(acc, fb, fa, lds, s, k2, k2, ptrs, ids, g);  // the A loads of stage st + 2
+  }
+
+  // Every per-lane value the main loop reads, marked as used: should the compiler have parked one of them in
+  // scratch memory around the caller's code, it reloads it (and waits for that load) here, and not inside the
+  // loop, where its wait would also wait for the direct-to-LDS loads in flight, stage after stage.
+  static __device__ __forceinline__ void pin(Source& s, Ptrs& ptrs, Geometry& g) {
+#pragma unroll
+    for (int q = 0; q < (A_KM ? 1 : NQ1); ++q) asm volatile("" : "+v"(s.a_row[q]));
+#pragma unroll
+    for (int q = 0; q < (B_KM ? 1 : NQ1); ++q) asm volatile("" : "+v"(s.b_row[q]));
+#pragma unroll
+    for (int q = 0; q < (A_KM ? NQ1 : 1); ++q) asm volatile("" : "+v"(ptrs.a[q]));
+#pragma unroll
+    for (int q = 0; q < (B_KM ? NQ1 : 1); ++q) asm volatile("" : "+v"(ptrs.b[q]));
+    if (A_KM) asm volatile("" : "+v"(s.a_km));
+    if (B_KM) asm volatile("" : "+v"(s.b_km));
+#pragma unroll
+    for (int x = 0; x < 4; ++x) asm volatile("" : "+v"(g.a_addr[x]), "+v"(g.b_addr[x]));
+  }
+
+  // acc = A . B over the whole reduction.  prefetch() with the same source must have been called and nothing
+  // may have touched the LDS ring since.  Ends with a barrier: the LDS may be reused right after.
+  static __device__ __forceinline__ void run(f32x16 (&acc)[WM][WN], Source& s, Ptrs& ptrs, int (&ids)[NQ1],
+                                             unsigned char* lds, Geometry& g) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const int nk = (s.k_total + BK - 1) / BK;
+    if (B_KM) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the row lookups of stage 1 sit behind the loads)
+#pragma unroll
+      for (int q = 0; q < NQ1; ++q) asm volatile("" : "+v"(ids[q]));
+    } else {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NQ1) : "memory");  // stage 0 landed, the A loads of stage 1 may be in flight
+    }
+    pin(s, ptrs, g);
+    __syncthreads();
+    Frags fa, fb;
+    read_all<0, 0>(fa, lds, g);
+
+    // two stages per trip, so that every LDS address is a lane constant plus an immediate; an odd last stage
+    // stands outside the loop (a branch inside it costs the register allocator its footing)
+#pragma unroll 1
+    for (int st = 0; st + 1 < nk; st += 2) {
+      stage<0>(acc, fa, fb, lds, s, st, ptrs, ids, g);
+      stage<1>(acc, fa, fb, lds, s, st + 1, ptrs, ids, g);
+    }
+    if (nk & 1) stage<0>(acc, fa, fb, lds, s, nk - 1, ptrs, ids, g);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch
+    __syncthreads();
+  }
+};
+
+}  // namespace cce

@@ -50,6 +50,12 @@ _SIGNATURES = {
         [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]
         + [_i64] * 4 + [_i64] * 3 + [_f32, _f32, _i32, _i32, _i32, _i32, _i64, _i64, _f32, _i32, _ptr],
     ),
+    "cce_backward_dense_workspace_bytes": (_i64, [_i64, _i64, _i64, _i32, _i64]),
+    "cce_backward_dense": (
+        _i32,
+        [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64]
+        + [_i64] * 4 + [_i64] * 3 + [_f32, _i32, _i32, _i64, _i64, _f32, _i32, _ptr],
+    ),
     "cce_backward_dz": (
         _i32,
         [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _i64, _i32]
@@ -117,3 +123,34 @@ def require_gpu_tensor(name: str, t: torch.Tensor) -> None:
 
 def current_stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+# Device timings for a benchmark: while a dict is set here, every launcher brackets its library calls with a
+# pair of events on the stream it launches on and appends the pair under its name.
+_timers: Optional[dict] = None
+
+
+def set_timers(timers: Optional[dict]) -> None:
+    global _timers
+    _timers = timers
+
+
+class timed:
+    """``with timed("name", device): lib.call(...)``: free when no benchmark is collecting."""
+
+    def __init__(self, name: str, device: torch.device):
+        self.name, self.device = name, device
+        self.start = None
+
+    def __enter__(self):
+        if _timers is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record(torch.cuda.current_stream(self.device))
+        return self
+
+    def __exit__(self, *exc):
+        if self.start is not None and _timers is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record(torch.cuda.current_stream(self.device))
+            _timers.setdefault(self.name, []).append((self.start, end))
+        return False

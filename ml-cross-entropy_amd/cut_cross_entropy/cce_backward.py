@@ -10,25 +10,10 @@ from cut_cross_entropy.cce_utils import filter_eps_or_none
 from cut_cross_entropy.utils import TensorInfo
 
 
-_DENSE_DZ_ELEMS = 1 << 27  # most elements of one dz chunk (256 MB in a 16-bit type)
-
-
-def _dense_chunk_classes(B: int, V: int, D: int) -> int:
-    """Classes per dz chunk of the unfiltered backward.  The dC product of a chunk is a [vc, D] GEMM whose
-    256 x 256 output tiles should fill the 256 compute units in whole rounds: measured at B = 8192, D = 2304
-    the library runs it at 1150 TFLOP/s with vc = 7168 (252 tiles) and at 730 with vc = 8192 (288 tiles).
-    Among the multiples of 256 in the upper half of what the dz buffer allows, take the best-filling one."""
-    top = max(256, min(8192, (_DENSE_DZ_ELEMS // max(B, 1)) // 256 * 256))
-    if top >= V:
-        return (V + 7) // 8 * 8
-    col_tiles = (D + 255) // 256
-    best, best_fill = top, -1.0
-    for vc in range(top, max(top // 2, 255), -256):
-        tiles = (vc // 256) * col_tiles
-        fill = tiles / (((tiles + 255) // 256) * 256)
-        if fill > best_fill + 1e-9:
-            best, best_fill = vc, fill
-    return best
+# Upper bound of the dz chunk buffer of the unfiltered backward (bytes).  The chunk is [B, vc] in the input type
+# with vc a multiple of 256 classes, at most 8192; the library picks the vc that fits.  A smaller buffer means
+# more, smaller chunks: less memory, launches that fill the GPU less evenly.
+DENSE_DZ_BYTES = 256 << 20
 
 # With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path pays for
 # the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
@@ -54,23 +39,6 @@ def _flagged_fraction(tile_max, lse, B, V, filter_eps) -> float:
     return float((bound >= math.log(filter_eps) - 0.01).float().mean().item())
 
 
-def _mm_fp32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """``a @ b`` of 16-bit operands with the fp32 accumulator handed back unrounded."""
-    try:
-        return torch.mm(a, b, out_dtype=torch.float32)
-    except (TypeError, RuntimeError):  # a build without the mixed-precision GEMM: rounded per chunk
-        return torch.mm(a, b).to(torch.float32)
-
-
-def _addmm_fp32(acc: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """``acc + a @ b`` in fp32 (acc fp32, a and b 16-bit), the addition inside the GEMM where the build has it."""
-    try:
-        return torch.addmm(acc, a, b, out_dtype=torch.float32, out=acc)
-    except (TypeError, RuntimeError):
-        acc += _mm_fp32(a, b)
-        return acc
-
-
 def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
     """The unfiltered backward runs as (dz kernel + library GEMMs) when nothing that is asked for is
     filtered and the layout suits the direct-to-LDS kernel."""
@@ -89,50 +57,31 @@ def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_gra
 
 def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
                     shift, target_offset, softcap):
-    """dE, dC, dBias of the unfiltered backward, one vocabulary chunk at a time: the kernel writes the
-    chunk's dz = d loss / d logits (never the logits), and the two products are library GEMMs
-    (reference: the products of cce_backward.py:262-302, there done with atomics inside the kernel).
-    dE is accumulated over the chunks in fp32; dC and dBias are complete per chunk."""
+    """dE, dC, dBias of the unfiltered backward: one call into the library, which walks the vocabulary in
+    chunks (dz of the chunk -> workspace, then the two products as hand-written MFMA kernels; reference:
+    cce_backward.py:170-302, there one kernel with atomics).  The workspace -- the dz chunk, plus an fp32
+    [B, D] accumulator when dE is wanted in the 16-bit input type -- is a torch allocation, so the allocator's
+    peak statistic sees it."""
     V, D = c.size(0), e.size(1)
-    vc = _dense_chunk_classes(B, V, D)
-    dz_buf = torch.empty((B * vc,), dtype=e.dtype, device=dev)
-    rows = valids.to(torch.int64) if valids is not None else None
-    e_rows = e if rows is None else e.index_select(0, rows)
-    de_acc = torch.zeros((B, D), dtype=torch.float32, device=dev) if de is not None else None
-    stream = _hip.current_stream_ptr(dev)
-    for v0 in range(0, V, vc):
-        n = min(vc, V - v0)
-        ldz = (n + 7) // 8 * 8
-        dz = dz_buf[: B * ldz].view(B, ldz)
-        c_chunk = c[v0 : v0 + n]
-        with torch.cuda.device(dev):
-            status = lib.cce_backward_dz(
-                e.data_ptr(), c_chunk.data_ptr(),
-                (bias.data_ptr() + v0 * bias.element_size()) if bias is not None else None,
-                lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
-                _hip.ptr(valids), targets.data_ptr(),
-                dz.data_ptr(), ldz, 0,
-                e.size(0), B, n, D,
-                e.stride(0), c.stride(0), c.stride(1),
-                float(grad_scale), int(shift), int(target_offset) + v0,
-                float(softcap) if softcap is not None else 0.0, code, stream,
-            )
-        _hip.check(status, "cce_backward_dz")
-        dzv = dz[:, :n]
-        if de_acc is not None:
-            de_acc = _addmm_fp32(de_acc, dzv, c_chunk)
-        if dc is not None:
-            if dc.dtype == torch.float32:
-                dc[v0 : v0 + n] = _mm_fp32(dzv.t(), e_rows)
-            else:
-                torch.mm(dzv.t(), e_rows, out=dc[v0 : v0 + n])
-        if dbias is not None:
-            dbias[v0 : v0 + n] = dzv.sum(dim=0, dtype=torch.float32)
-    if de is not None:
-        if rows is None:
-            de.copy_(de_acc)
-        else:
-            de.index_copy_(0, rows, de_acc.to(de.dtype))
+    de_in_ws = de is not None and de.dtype != torch.float32
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_in_ws else 0, DENSE_DZ_BYTES)
+    workspace = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
+    ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
+    with torch.cuda.device(dev), _hip.timed("backward_dense", dev):
+        status = lib.cce_backward_dense(
+            e.data_ptr(), c.data_ptr(), _hip.ptr(bias),
+            lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
+            _hip.ptr(valids), targets.data_ptr(),
+            _hip.ptr(de), _hip.ptr(dc), _hip.ptr(dbias),
+            ws_ptr, ws_bytes,
+            e.size(0), B, V, D,
+            e.stride(0), c.stride(0), c.stride(1),
+            float(grad_scale), 1 if (de is not None and de.dtype == torch.float32) else 0,
+            1 if (dc is not None and dc.dtype == torch.float32) else 0,
+            int(shift), int(target_offset),
+            float(softcap) if softcap is not None else 0.0, code, _hip.current_stream_ptr(dev),
+        )
+    _hip.check(status, "cce_backward_dense")
 
 
 def cce_backward_kernel(
@@ -214,13 +163,14 @@ def cce_backward_kernel(
         dense = _flagged_fraction(tile_max, lse.to(torch.float32), n_valid, c.size(0), float(filter_eps)) \
             > DENSE_WHEN_FLAGGED_ABOVE / -(-e.size(1) // _OWNERSHIP_SLICE_COLS)
     if dense:
-        # every GEMM of the dense path accumulates in fp32 internally and each output element is written
-        # once (dC, dBias) or summed in a separate fp32 buffer (dE): no fp32 gradient buffers are needed
+        # the products of the dense path accumulate in fp32 registers and each output element is written once
+        # (dC, dBias) or summed over the chunks in an fp32 workspace (dE): no fp32 gradient buffers are needed
         de_dtype, dc_dtype = e_info.dtype, c_info.dtype
     de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
     dc = None
     if c_info.requires_grad:
-        dc = torch.zeros_like(c, dtype=dc_dtype)
+        # the dense path writes every element of dC; the ownership kernels leave untouched rows to the zeros
+        dc = torch.empty_like(c, dtype=dc_dtype) if dense else torch.zeros_like(c, dtype=dc_dtype)
         if dc.stride() != c.stride():
             # a view with gaps between its rows or columns (zeros_like packs those): the kernels address C and
             # dC with one pair of strides, so dC gets the layout of c, or c is packed if its elements overlap
@@ -271,7 +221,7 @@ def cce_backward_kernel(
     elif B > 0 and wanted:
         ws_bytes = lib.cce_backward_workspace_bytes(B, c.size(0), e.size(1))
         workspace = torch.empty((max(ws_bytes, 8) // 8 + 1,), dtype=torch.int64, device=dev)
-        with torch.cuda.device(dev):
+        with torch.cuda.device(dev), _hip.timed("backward_sparse", dev):
             status = lib.cce_backward(
                 e.data_ptr(), c.data_ptr(), _hip.ptr(bias),
                 lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),

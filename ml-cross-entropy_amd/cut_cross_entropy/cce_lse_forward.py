@@ -53,7 +53,7 @@ def lse_forward(
 
     ws_bytes = lib.cce_lse_forward_workspace_bytes(B, V, D)
     workspace = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.int64, device=e.device)
-    with torch.cuda.device(e.device):
+    with torch.cuda.device(e.device), _hip.timed("lse_forward", e.device):
         status = lib.cce_lse_forward(
             e.data_ptr(), c.data_ptr(), _hip.ptr(bias), _hip.ptr(valids),
             lse.data_ptr(), _hip.ptr(logit_avg), _hip.ptr(tile_max),

@@ -221,6 +221,98 @@ def test_backward_dz_abi(dtype, softcap, has_bias, with_dlse, shape):
         assert_no_worse(gt[2], ref[2], dz_full.sum(0), tol, "dBias", rel)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("softcap", [None, 20.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("fp32_out", [False, True])
+@pytest.mark.parametrize("shape,dz_budget", [((256, 512, 128), 0), ((255, 507, 64), 0), ((700, 1300, 192), 0),
+                                             ((300, 1100, 320), 1 << 30), ((520, 2100, 576), 520 * 768 * 2)])
+def test_backward_dense_abi(dtype, softcap, has_bias, fp32_out, shape, dz_budget):
+    """cce_backward_dense (dz chunks + hand-written dE / dC products, one call) vs the closed-form dense
+    gradients: several chunks (smallest workspace), one chunk (large workspace), ragged rows, classes and
+    columns, rows gathered through valids, upstream d_lse."""
+    from oracle import dense_lce
+
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D = shape
+    e, c, t, bias = make_inputs(N, V, D, dtype, seed=6, bias=has_bias, invalid_frac=0.2)
+    valids = dense_lce.build_flat_valids(t, IGNORE_INDEX, 0)
+    B = valids.numel()
+    g = torch.Generator().manual_seed(13)
+    d_out = torch.randn((N,), generator=g)
+    d_lse = torch.randn((N,), generator=g) * 0.1
+    rows = valids.long()
+    lse = dense_lce.dense_lse(e[rows], c, bias, softcap, torch.float64)
+    gt = dense_lce.dense_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, torch.float64)
+    ref = autograd_grads(e, c, t, valids, d_out * 0.5, d_lse, bias, softcap, 0, dtype)
+
+    ed, cd, td, vd = e.to(dev), c.to(dev), t.to(dev), valids.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    lsed, dod, dld = lse.float().to(dev), d_out.float().to(dev), d_lse.float().to(dev)
+    gdt = torch.float32 if fp32_out else dtype
+    de = torch.zeros((N, D), dtype=gdt, device=dev)
+    dc = torch.full((V, D), float("nan"), dtype=gdt, device=dev)  # written, not accumulated
+    db = torch.zeros((V,), dtype=torch.float32, device=dev) if bias is not None else None
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 0 if fp32_out else 1, dz_budget)
+    ws = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
+    ws_ptr = (ws.data_ptr() + 255) // 256 * 256
+    p = lambda x: x.data_ptr() if x is not None else None
+    st = lib.cce_backward_dense(
+        p(ed), p(cd), p(bd), p(lsed), p(dod), 0, p(dld), p(vd), p(td),
+        p(de), p(dc), p(db), ws_ptr, ws_bytes,
+        N, B, V, D, ed.stride(0), cd.stride(0), cd.stride(1),
+        0.5, 1 if fp32_out else 0, 1 if fp32_out else 0, 0, 0,
+        softcap or 0.0, 0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream)
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    tol, rel = 2e-3, 1e-2
+    assert_no_worse(gt[0], ref[0], de.cpu(), tol, "dE", rel)
+    assert_no_worse(gt[1], ref[1], dc.cpu(), tol, "dC", rel)
+    if has_bias:
+        assert_no_worse(gt[2], ref[2], db.cpu(), tol, "dBias", rel)
+    ignored = torch.ones(N, dtype=torch.bool)
+    ignored[rows] = False
+    assert (de.cpu()[ignored] == 0).all()
+
+
+def test_backward_dense_ignores_non_finite_values_it_must_not_read():
+    """Rows of e that are not valid and the reduction tails of the product tiles must not leak into the
+    gradients: an ignored row full of inf / nan (and such a row as row 0, where absent rows used to point)
+    leaves every gradient finite."""
+    from oracle import dense_lce
+
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D, dtype = 203, 333, 64, torch.bfloat16
+    e, c, t, _ = make_inputs(N, V, D, dtype, seed=8)
+    t[0] = IGNORE_INDEX
+    t[77] = IGNORE_INDEX
+    e[0] = float("inf")
+    e[77] = float("nan")
+    valids = dense_lce.build_flat_valids(t, IGNORE_INDEX, 0)
+    B = valids.numel()
+    rows = valids.long()
+    lse = dense_lce.dense_lse(e[rows], c, None, None, torch.float64)
+    d_out = torch.ones((N,))
+    gt = dense_lce.dense_grads(e[rows], c, t[rows], None, d_out[rows], None, None, None, 0, torch.float64)
+    ed, cd, td, vd = e.to(dev), c.to(dev), t.to(dev), valids.to(dev)
+    lsed, dod = lse.float().to(dev), d_out.to(dev)
+    de = torch.zeros((N, D), dtype=dtype, device=dev)
+    dc = torch.zeros((V, D), dtype=dtype, device=dev)
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1, 0)
+    ws = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
+    st = lib.cce_backward_dense(
+        ed.data_ptr(), cd.data_ptr(), None, lsed.data_ptr(), dod.data_ptr(), 0, None, vd.data_ptr(), td.data_ptr(),
+        de.data_ptr(), dc.data_ptr(), None, (ws.data_ptr() + 255) // 256 * 256, ws_bytes,
+        N, B, V, D, D, D, 1, 1.0, 0, 0, 0, 0, 0.0, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    assert torch.isfinite(dc).all() and torch.isfinite(de[vd.long()]).all()
+    assert torch.allclose(dc.cpu().double(), gt[1], atol=2e-2, rtol=2e-2)
+    assert torch.allclose(de.cpu().double()[rows], gt[0], atol=2e-2, rtol=2e-2)
+
+
 def test_backward_dz_rejects_layouts_it_cannot_stream():
     lib = _lib()
     dev = torch.device("cuda:0")
