@@ -156,6 +156,17 @@ int cce_backward(const void* e, const void* c, const void* bias,
                  int64_t shift, int64_t target_offset,
                  float softcap, int dtype, void* stream);
 
+/*
+ * count += number of cells of the forward statistic (CCE_STAT_ROWS x CCE_STAT_COLS) whose bound
+ * exp(tile_max - min lse of the cell's rows) reaches filter_eps, i.e. the cells cce_backward has to recompute.
+ * The fraction count / cce_tile_stat_elems(b, v) tells a caller whether filtering can pay at all (near-uniform
+ * soft-max distributions flag almost every cell; the unfiltered cce_backward_dense is then faster and exact).
+ * The reference has no counterpart: its kernel meets every tile anyway (cut_cross_entropy/cce_backward.py:170-216).
+ *   tile_max, lse  as written by cce_lse_forward for the same b, v;   count  one uint64, accumulated into
+ */
+int cce_count_flagged_cells(const float* tile_max, const float* lse, int64_t b, int64_t v, float filter_eps,
+                            uint64_t* count, void* stream);
+
 /* The logit gradient of one vocabulary chunk, written out, for the unfiltered backward.
  *
  * Restates the first half of the Triton backward body (cut_cross_entropy/cce_backward.py:

@@ -1,7 +1,7 @@
 // Version and status text of the C ABI.
 #include "cce_common.h"
 
-extern "C" int cce_version(void) { return 4; }
+extern "C" int cce_version(void) { return 5; }
 
 extern "C" const char* cce_error_string(int status) {
   switch (status) {

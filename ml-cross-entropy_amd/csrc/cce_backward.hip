@@ -606,9 +606,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
 // Stage layout: 256-byte rows (128 columns), 16-byte chunks XOR-swizzled with (row & 15); one load
 // instruction of a wave fills 1 KB = 4 rows, lane l -> row (l >> 4), chunk slot (l & 15).  Other-side
 // block b = q * 4 + wave holds rows [4 b, 4 b + 4) of the 128-row virtual cell; own-side likewise for
-// its 32 rows.  A row id of -1 (no row) is fetched from row 0 of the matrix: the values are finite
-// and only ever meet a dz of exactly zero.
+// its 32 rows.  A row id of -1 (no row: past the last valid row or the last class) is fetched from a
+// line of zeros, whatever the stage: its products are exactly zero and no non-finite value of another
+// row of the matrices can leak into real rows through it.
 // ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) uint16_t g_owner_zero_line[128];  // never written
+
 constexpr int kFCols = 128;
 constexpr int kFRowBytes = 256;
 constexpr int kFOtherBytes = 128 * kFRowBytes;      // 32 KB
@@ -730,11 +733,15 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
   const int* own_ids = IS_DE ? meta.row : sOwnCid;
 
   // own-side load pointers (2 per wave and stage), fixed for the whole kernel
+  // (a row that does not exist points at the line of zeros and does not advance with the stage)
+  const uint16_t* zero_chunk = g_owner_zero_line + (lane & 15) * 8;
   const uint16_t* own_ptr[2];
+  int own_step[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
     const int id = own_ids[4 * (q * 4 + wave) + (lane >> 4)];
-    own_ptr[q] = own_base + static_cast<int64_t>(id < 0 ? 0 : id) * own_sr + lane_chunk;
+    own_ptr[q] = (id < 0) ? zero_chunk : own_base + static_cast<int64_t>(id) * own_sr + lane_chunk;
+    own_step[q] = (id < 0) ? 0 : 1;
   }
 
   // wave w owns columns [32 w, 32 w + 32) of every 128-column chunk
@@ -855,10 +862,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 
       // other-side load pointers of this trip (8 per wave and stage)
       const uint16_t* other_ptr[8];
+      uint32_t other_live = 0u;  // bit q: load q fetches a real row (advances with the stage)
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
         const int id = other_ids[4 * (q * 4 + wave) + (lane >> 4)];
-        other_ptr[q] = other_base + static_cast<int64_t>(id < 0 ? 0 : id) * other_sr + lane_chunk;
+        other_ptr[q] = (id < 0) ? zero_chunk : other_base + static_cast<int64_t>(id) * other_sr + lane_chunk;
+        other_live |= (id < 0 ? 0u : 1u) << q;
       }
       // Entries are packed at the front of a trip; the rows of absent ones are not fetched (loads
       // 2 e and 2 e + 1 of a wave belong to entry e), so a short trip moves proportionally less data.
@@ -872,10 +881,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         const unsigned base = lds_base + slot * slot_bytes;
 #pragma unroll
         for (int q = 0; q < 8; ++q)
-          if ((entries >> (q >> 1)) & 1u) lds_dma16(other_ptr[q] + col0, base + (q * 4 + wave) * 1024);
+          if ((entries >> (q >> 1)) & 1u)
+            lds_dma16(other_ptr[q] + (((other_live >> q) & 1u) ? col0 : 0), base + (q * 4 + wave) * 1024);
         if (with_own) {
 #pragma unroll
-          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + col0, base + own_off + (q * 4 + wave) * 1024);
+          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + (own_step[q] ? col0 : 0), base + own_off + (q * 4 + wave) * 1024);
         }
       };
 
@@ -1092,9 +1102,48 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
   }
 }
 
+// Number of cells of the forward statistic (32 rows x 32 classes) whose bound exp(max logit - min lse of the 32
+// rows) reaches eps: the cells the ownership kernels have to recompute.  One workgroup per row group.
+__global__ __launch_bounds__(256) void flagged_cells_kernel(const float* tile_max, const float* lse, int64_t b, int stat_cols,
+                                                            float log_eps, unsigned long long* count) {
+  __shared__ float s_min;
+  __shared__ unsigned int s_part[4];
+  const int tg = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave == 0) {
+    const int64_t i = static_cast<int64_t>(tg) * 32 + lane;
+    const float mn = wave_min((lane < 32 && i < b) ? lse[i] : INFINITY);
+    if (lane == 0) s_min = mn;
+  }
+  __syncthreads();
+  const float min_lse = s_min;
+  const float* row = tile_max + static_cast<int64_t>(tg) * stat_cols;
+  unsigned int n = 0;
+  for (int j = threadIdx.x; j < stat_cols; j += 256) n += (row[j] - min_lse >= log_eps) ? 1u : 0u;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) n += __shfl_xor(n, off, 64);
+  if (lane == 0) s_part[wave] = n;
+  __syncthreads();
+  if (threadIdx.x == 0) atomicAdd(count, static_cast<unsigned long long>(s_part[0] + s_part[1] + s_part[2] + s_part[3]));
+}
+
 }  // namespace cce
 
 using namespace cce;
+
+extern "C" int cce_count_flagged_cells(const float* tile_max, const float* lse, int64_t b, int64_t v, float filter_eps,
+                                       uint64_t* count, void* stream_) {
+  if (b < 0 || v <= 0 || !(filter_eps > 0.0f)) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0) return CCE_OK;
+  if (tile_max == nullptr || lse == nullptr || count == nullptr) return CCE_ERR_INVALID_ARGUMENT;
+  const int64_t ntg = (b + CCE_STAT_ROWS - 1) / CCE_STAT_ROWS;
+  if (ntg >= (int64_t(1) << 31) || v >= (int64_t(1) << 31) - 512) return CCE_ERR_INVALID_ARGUMENT;
+  const int stat_cols = static_cast<int>((v + CCE_STAT_COLS - 1) / CCE_STAT_COLS);
+  hipLaunchKernelGGL(flagged_cells_kernel, dim3(static_cast<unsigned>(ntg)), dim3(256), 0, static_cast<hipStream_t>(stream_),
+                     tile_max, lse, b, stat_cols, logf(filter_eps) - 0.01f,
+                     reinterpret_cast<unsigned long long*>(count));
+  return status_from_hip(hipGetLastError());
+}
 
 static int64_t bit_words_for(int64_t v) { return ((v + 31) / 32 + 31) / 32; }
 

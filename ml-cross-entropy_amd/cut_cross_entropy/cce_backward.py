@@ -1,6 +1,7 @@
 """Launcher of the fused backward kernel
 (reference: cut_cross_entropy/cce_backward.py:346-521)."""
 
+import threading
 from typing import Optional, Tuple
 
 import torch
@@ -19,24 +20,69 @@ DENSE_DZ_BYTES = 256 << 20
 # the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
 # statistic can hold a probability above filter_eps for E [8192, 2304] x C [256000, 2304], and at 0.083 for
 # E [16384, 4096] x C [128256, 4096], where a workgroup of the ownership kernels covers D in two slices and
-# recomputes its logits for each.  Above DENSE_WHEN_FLAGGED_ABOVE / slices (the fraction is read off the
-# forward's statistic with one small reduction and one host read) the backward runs unfiltered; an
+# recomputes its logits for each.  Above DENSE_WHEN_FLAGGED_ABOVE / slices the backward runs unfiltered; an
 # unfiltered gradient is the exact one, so nothing is lost.  None switches the test off.
+#
+# The fraction is measured on the device (cce_count_flagged_cells over the forward's statistic) and read on the
+# host WITHOUT waiting for the device: every filtered backward enqueues the count and an asynchronous copy of
+# it to pinned host memory, and uses the most recent count that has arrived -- normally that of the step
+# before.  The soft-max distribution of a model moves slowly, so a decision that lags one step is as good;
+# the first backward of a shape has no count yet and takes the ownership kernels (always correct, slower when
+# the soft-max is flat).  FILTERED_BACKWARD_PATH pins the choice: "sparse" or "dense" instead of "auto".
 DENSE_WHEN_FLAGGED_ABOVE = 0.17
+FILTERED_BACKWARD_PATH = "auto"
 _OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
 
-def _flagged_fraction(tile_max, lse, B, V, filter_eps) -> float:
-    """Fraction of the cells of the forward statistic (32 rows x ``STAT_COLS`` classes) whose bound
-    exp(max logit - min lse) reaches filter_eps."""
-    import math
+class _FlaggedMonitor:
+    """Latest measured fraction of flagged cells for one (device, V, D, dtype), read without a host wait."""
 
-    ntg, nvc = (B + 31) // 32, (V + _hip.STAT_COLS - 1) // _hip.STAT_COLS
-    lse_pad = torch.full((ntg * 32,), float("inf"), dtype=torch.float32, device=lse.device)
-    lse_pad[:B] = lse
-    lse_min = lse_pad.view(ntg, 32).min(dim=1).values
-    bound = tile_max.view(ntg, nvc) - lse_min[:, None]
-    return float((bound >= math.log(filter_eps) - 0.01).float().mean().item())
+    def __init__(self, device: torch.device):
+        self.counter = torch.zeros((1,), dtype=torch.int64, device=device)
+        self.host = torch.zeros((1,), dtype=torch.int64, pin_memory=True)
+        self.event = torch.cuda.Event()
+        self.pending_cells = 0   # cells of the measurement in flight (0: none)
+        self.fraction: Optional[float] = None
+
+    def poll(self) -> Optional[float]:
+        if self.pending_cells and self.event.query():
+            self.fraction = int(self.host[0]) / self.pending_cells  # pinned host memory: a plain read
+            self.pending_cells = 0
+        return self.fraction
+
+    def measure(self, lib, tile_max, lse, B: int, V: int, filter_eps: float, dev: torch.device) -> None:
+        if self.pending_cells or torch.cuda.is_current_stream_capturing():
+            return  # one measurement in flight at a time; none inside a graph capture
+        self.counter.zero_()
+        with torch.cuda.device(dev):
+            status = lib.cce_count_flagged_cells(tile_max.data_ptr(), lse.data_ptr(), B, V, float(filter_eps),
+                                                 self.counter.data_ptr(), _hip.current_stream_ptr(dev))
+        _hip.check(status, "cce_count_flagged_cells")
+        self.host.copy_(self.counter, non_blocking=True)
+        self.event.record(torch.cuda.current_stream(dev))
+        self.pending_cells = lib.cce_tile_stat_elems(B, V)
+
+
+_monitors: dict = {}
+_monitors_lock = threading.Lock()
+
+
+def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, filter_eps: float, dtype, dev) -> bool:
+    """The dense / sparse choice of a filtered backward; never waits for the device."""
+    if FILTERED_BACKWARD_PATH != "auto":
+        return FILTERED_BACKWARD_PATH == "dense"
+    if DENSE_WHEN_FLAGGED_ABOVE is None:
+        return False
+    key = (dev.index, V, D, dtype)
+    with _monitors_lock:
+        mon = _monitors.get(key)
+        if mon is None:
+            if torch.cuda.is_current_stream_capturing():
+                return False  # nothing may be allocated for a new shape inside a capture
+            mon = _monitors[key] = _FlaggedMonitor(dev)
+        fraction = mon.poll()
+        mon.measure(lib, tile_max, lse, B, V, filter_eps, dev)
+    return fraction is not None and fraction > DENSE_WHEN_FLAGGED_ABOVE / -(-D // _OWNERSHIP_SLICE_COLS)
 
 
 def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
@@ -156,12 +202,11 @@ def cce_backward_kernel(
     dense = _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad,
                             bias is not None and bias_info is not None and bias_info.requires_grad,
                             filter_eps, filter_e_grad, filter_c_grad)
-    if (not dense and DENSE_WHEN_FLAGGED_ABOVE is not None and tile_max is not None and filter_eps is not None
-            and filter_eps > 0 and lse.numel() > 0
+    if (not dense and tile_max is not None and filter_eps is not None and filter_eps > 0 and lse.numel() > 0
             and _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad, False, None, False, False)):
         n_valid = valids.size(0) if valids is not None else e.size(0)
-        dense = _flagged_fraction(tile_max, lse.to(torch.float32), n_valid, c.size(0), float(filter_eps)) \
-            > DENSE_WHEN_FLAGGED_ABOVE / -(-e.size(1) // _OWNERSHIP_SLICE_COLS)
+        dense = _filtered_backward_runs_dense(lib, tile_max, lse, n_valid, c.size(0), e.size(1), float(filter_eps),
+                                              e.dtype, dev)
     if dense:
         # the products of the dense path accumulate in fp32 registers and each output element is written once
         # (dC, dBias) or summed over the chunks in an fp32 workspace (dE): no fp32 gradient buffers are needed

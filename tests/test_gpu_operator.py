@@ -208,8 +208,10 @@ def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids
 
 def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     """Near-uniform soft-max over few classes: every cell's bound exp(max logit - min lse) is above
-    filter_eps, so the backward runs unfiltered (and is then exact); with the switch off the
-    ownership kernels run.  Peaked soft-max over many classes: the sparse kernels stay."""
+    filter_eps, so the backward runs unfiltered (and is then exact) -- from the second step on: the count of
+    flagged cells is read without waiting for the device, so a step uses the count of the step before, and the
+    first step of a shape runs the ownership kernels.  With the switch off the ownership kernels run.  Peaked
+    soft-max over many classes: the sparse kernels stay."""
     from cut_cross_entropy import cce_backward as bw
     from cut_cross_entropy import linear_cross_entropy
     from oracle import dense_lce
@@ -217,29 +219,133 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     calls = []
     real = bw._dense_backward
     monkeypatch.setattr(bw, "_dense_backward", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    monkeypatch.setattr(bw, "_monitors", {})
 
     e, c, t, _ = make_inputs(512, 2048, 128, torch.bfloat16, seed=4, planted=False, c_std=0.05)
     ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
-    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
-    assert len(calls) == 1
     e64, c64 = e.double().requires_grad_(True), c.double().requires_grad_(True)
     dense_lce.dense_linear_cross_entropy(e64, c64, t)[0].backward()
-    assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=2e-2 / 512, rtol=2e-2)
-    assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=2e-2 / 512, rtol=2e-2)
+    for step in range(2):
+        ed.grad = cd.grad = None
+        linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+        torch.cuda.synchronize()
+        assert len(calls) == step  # step 0: no count yet -> ownership kernels; step 1: dense
+        tol = 2e-2 if step == 1 else 5e-2  # the filtered gradient of step 0 differs by the dropped sub-tiles
+        assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=tol / 512, rtol=tol)
+        assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=tol / 512, rtol=tol)
 
     monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", None)
     ed.grad = cd.grad = None
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     assert len(calls) == 1
-
     monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", 0.17)
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "sparse")
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    assert len(calls) == 1
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "dense")
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    assert len(calls) == 2
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "auto")
+
     g = torch.Generator().manual_seed(1)
     c2 = (torch.randn((65536, 128), generator=g) * 0.5).to(torch.bfloat16)  # 512 cells per row group, <= 32 hold a target
     t2 = torch.randint(0, 65536, (512,), generator=g)
     e2 = (c2[t2].float() * 4).to(torch.bfloat16)  # each row points at its own class: a peaked soft-max
     ed2, cd2 = e2.cuda().requires_grad_(True), c2.cuda().requires_grad_(True)
-    linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
-    assert len(calls) == 1
+    for _ in range(2):
+        linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
+        torch.cuda.synchronize()
+    assert len(calls) == 2
+
+
+@pytest.mark.parametrize("impl", ["cce", "cce_exact"])
+def test_backward_never_waits_for_the_device(impl):
+    """No host synchronisation between the entry of backward() and its return (the reference's backward has
+    none either, cce.py:166-235): torch's sync debug mode turns any .item() / .cpu() / nonzero into an error."""
+    from cut_cross_entropy import linear_cross_entropy
+
+    e, c, t, _ = make_inputs(512, 2048, 128, torch.bfloat16, seed=5, planted=False, c_std=0.05)
+    ed, cd, td = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True), t.cuda()
+    for _ in range(3):  # first step: new monitor, kernel attributes; later steps: the steady state
+        ed.grad = cd.grad = None
+        loss = linear_cross_entropy(ed, cd, td, softcap=20.0, impl=impl)
+        torch.cuda.synchronize()
+        torch.cuda.set_sync_debug_mode("error")
+        try:
+            loss.backward()
+        finally:
+            torch.cuda.set_sync_debug_mode("default")
+        torch.cuda.synchronize()
+    assert torch.isfinite(ed.grad).all() and torch.isfinite(cd.grad).all()
+
+
+@pytest.mark.parametrize("impl,path", [("cce", "sparse"), ("cce", "dense"), ("cce_exact", "auto")])
+def test_operator_backward_replays_in_a_hip_graph(monkeypatch, impl, path):
+    """loss.backward() of the operator captured in a HIP graph (the forward runs eagerly on the capture stream:
+    it reads the number of valid rows on the host, as the reference does) and replayed on new contents of e and
+    c: every replay gives the gradients of an eager backward on the same contents."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", path)
+    e0, c0, t0, _ = make_inputs(384, 3000, 128, torch.bfloat16, seed=6, planted=True)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        ed, cd, td = e0.cuda().requires_grad_(True), c0.cuda().requires_grad_(True), t0.cuda()
+
+        def eager_grads():
+            ed.grad = cd.grad = None
+            linear_cross_entropy(ed, cd, td, softcap=20.0, impl=impl).backward()
+            return ed.grad.clone(), cd.grad.clone()
+
+        eager_grads()  # loads the library, sets kernel attributes outside the capture
+        ed.grad = cd.grad = None
+        loss = linear_cross_entropy(ed, cd, td, softcap=20.0, impl=impl)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        loss.backward(retain_graph=True)
+    de_static, dc_static = ed.grad, cd.grad
+    # The saved log-sum-exp belongs to the captured forward, so the replays keep e and c; what a replay must
+    # reproduce is the whole backward, into buffers that were overwritten in between.
+    with torch.cuda.stream(side):
+        ed.grad = cd.grad = None
+        linear_cross_entropy(ed, cd, td, softcap=20.0, impl=impl).backward()
+        want_de, want_dc = ed.grad.clone(), cd.grad.clone()
+    side.synchronize()
+    for rep in range(3):
+        de_static.fill_(7.0)
+        dc_static.fill_(7.0)
+        junk = torch.randn((1 << 22,), device="cuda")  # eager work and a synchronisation between the replays
+        junk.sum().item()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(de_static, want_de) and torch.equal(dc_static, want_dc), rep
+
+
+def test_rows_that_do_not_exist_read_as_zeros_in_the_ownership_kernels(monkeypatch):
+    """An ignored row of e full of inf sitting in row 0, a number of valid rows and of classes that are not
+    multiples of 32: the padding rows of the last row group and class group must read as zeros (a masked load
+    in the reference), not as row 0, whose inf times a zero dz would poison the gradients of real rows."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "sparse")
+    N, V, D = 200, 1001, 128  # D % 128 == 0: the fast ownership kernels
+    e, c, t, _ = make_inputs(N, V, D, torch.bfloat16, seed=7, planted=True)
+    t[0] = IGNORE_INDEX
+    e[0] = float("inf")
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert torch.isfinite(cd.grad).all(), "dC poisoned by a row that is not part of the batch"
+    assert torch.isfinite(ed.grad[1:]).all() and (ed.grad[0] == 0).all()
+    e64 = e[1:].double().requires_grad_(True)
+    c64 = c.double().requires_grad_(True)
+    dense_lce.dense_linear_cross_entropy(e64, c64, t[1:])[0].backward()
+    assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=5e-2 / 199, rtol=5e-2)
+    assert torch.allclose(ed.grad[1:].double().cpu(), e64.grad, atol=5e-2 / 199, rtol=5e-2)
 
 
 @pytest.fixture
@@ -297,6 +403,39 @@ def test_fp32_inputs_match_fp64_oracle(highest_matmul_precision, softcap, has_bi
     if shift:
         ignored = torch.cat([ignored[shift:], torch.ones(shift, dtype=torch.bool)])
     assert (ed.grad.cpu()[ignored] == 0).all()
+
+
+@pytest.mark.parametrize("shape", [(1, 33, 8), (1, 40, 8), (2, 33, 8), (1, 63, 8), (1, 33, 16)])
+@pytest.mark.parametrize("impl", ["cce", "cce_exact"])
+def test_fp32_one_row_peaked_soft_max(highest_matmul_precision, shape, impl):
+    """One or two rows, fewer than 64 classes, 8 columns, fp32, each row pointing at its own class: the loss
+    -log p_target is close to zero (p_target ~ 0.99) while the log-sum-exp and the target logit it is the
+    difference of are ~ 6, and the gradients carry the factor (1 - p_target).  In fp32 both therefore come with an
+    ABSOLUTE error of a few ulp of the log-sum-exp (|lse| 2^-23), whatever the implementation: the reference forms
+    nll = lse - logit in fp32 as well (cce.py:127-131).  A purely relative bound misreads that as an error (the
+    bound of 2e-5 on the loss is missed by 6x at |loss| = 0.01 with an absolute error of 1e-6); the bound here is
+    relative to the quantities the result is computed from."""
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    N, V, D = shape
+    g = torch.Generator().manual_seed(104)
+    c = torch.randn((V, D), generator=g) * (2.0 / D) ** 0.5
+    t = torch.randint(0, V, (N,), generator=g)
+    e = 3.0 * c[t] + 0.3 * torch.randn((N, D), generator=g)
+    e64, c64 = e.double().requires_grad_(True), c.double().requires_grad_(True)
+    want, want_lse = dense_lce.dense_linear_cross_entropy(e64, c64, t, return_lse=True)
+    want.backward()
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    loss, lse = linear_cross_entropy(ed, cd, t.cuda(), impl=impl, return_lse=True)
+    loss.backward()
+    ulp = 2.0**-23 * want_lse.abs().max().item()
+    assert abs(loss.item() - want.item()) <= 1e-5 * abs(want.item()) + 4 * ulp
+    assert torch.allclose(lse.cpu().double(), want_lse.detach(), rtol=1e-6, atol=4 * ulp)
+    # d nll / d logit = p - onehot is known to 4 ulp of the log-sum-exp; the products scale it by |c| resp. |e|
+    for got, ref, other in ((ed.grad, e64.grad, c), (cd.grad, c64.grad, e)):
+        bound = 5e-4 * ref.abs().max().item() + 8 * ulp * other.abs().max().item() / N
+        assert (got.cpu().double() - ref).abs().max().item() <= bound
 
 
 def test_fp32_mean_and_lse_and_shard(highest_matmul_precision):
