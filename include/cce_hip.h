@@ -53,6 +53,10 @@ extern "C" {
 /* Library ABI version (bumped when a signature below changes). */
 int cce_version(void);
 
+/* First 16 hex digits of the SHA-256 over the library's sources as they were when it was built (the order of
+ * csrc/Makefile: SRCS, then HDRS); lets a binding refuse a library that is older than the sources beside it. */
+const char* cce_source_hash(void);
+
 /* Human-readable text for a status returned by any function below. */
 const char* cce_error_string(int status);
 

@@ -3,6 +3,11 @@
 
 extern "C" int cce_version(void) { return 5; }
 
+#ifndef CCE_SOURCE_HASH
+#define CCE_SOURCE_HASH "unknown"
+#endif
+extern "C" const char* cce_source_hash(void) { return CCE_SOURCE_HASH; }
+
 extern "C" const char* cce_error_string(int status) {
   switch (status) {
     case CCE_OK: return "success";

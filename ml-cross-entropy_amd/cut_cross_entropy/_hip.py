@@ -28,6 +28,7 @@ _i64, _i32, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 _SIGNATURES = {
     "cce_version": (ctypes.c_int, []),
     "cce_error_string": (ctypes.c_char_p, [_i32]),
+    "cce_source_hash": (ctypes.c_char_p, []),
     "cce_tile_stat_elems": (_i64, [_i64, _i64]),
     "cce_lse_forward_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "cce_backward_workspace_bytes": (_i64, [_i64, _i64, _i64]),
@@ -69,6 +70,29 @@ def lib_path() -> str:
     return _LIB_PATH
 
 
+_CSRC = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "csrc"))
+
+
+def _hash_of_sources() -> Optional[str]:
+    """The hash csrc/Makefile builds into the library, recomputed from the files in the tree (None when the
+    sources are not there, e.g. an installed copy of the package)."""
+    import hashlib
+    import re
+
+    try:
+        text = open(os.path.join(_CSRC, "Makefile")).read()
+        names = []
+        for var in ("SRCS", "HDRS"):
+            names += re.search(rf"^{var} := (.*)$", text, flags=re.M).group(1).split()
+        digest = hashlib.sha256()
+        for name in names:
+            with open(os.path.join(_CSRC, name), "rb") as f:
+                digest.update(f.read())
+        return digest.hexdigest()[:16]
+    except (OSError, AttributeError):
+        return None
+
+
 def load() -> ctypes.CDLL:
     """Load the HIP library once; raise RuntimeError with build instructions if absent."""
     global _lib
@@ -91,6 +115,12 @@ def load() -> ctypes.CDLL:
         if lib.cce_version() != ABI_VERSION:
             raise RuntimeError(
                 f"libcce_hip.so ABI version {lib.cce_version()} does not match the Python binding ({ABI_VERSION}); rebuild it"
+            )
+        built_from, sources = lib.cce_source_hash().decode(), _hash_of_sources()
+        if sources is not None and built_from != sources:
+            raise RuntimeError(
+                f"libcce_hip.so was built from other sources (hash {built_from}) than those in {_CSRC} (hash {sources}): "
+                "rebuild it with `make -C ml-cross-entropy_amd/csrc`"
             )
         _lib = lib
     return _lib

@@ -24,6 +24,7 @@ from cut_cross_entropy.utils import TensorInfo, _build_flat_valids, _handle_eps,
 from cut_cross_entropy.vocab_parallel.utils import VocabParallelOptions, require_single_rank
 
 _REDUCTIONS = ("mean", "sum", "none")
+_D_MULTIPLE = 128  # columns per stage of the fast backward kernels
 
 
 @dataclass(frozen=True)
@@ -218,8 +219,15 @@ def cce_linear_cross_entropy(
     # order of magnitude slower than one packing copy (0.3 ms for 1.2 GB); autograd carries dC back through it.
     if not _streamable(c):
         c = c.contiguous()
-    targets = targets.contiguous()
+    # The direct-to-LDS kernels stream whole 128-column stages.  A width that is no multiple of 128 (D = 72,
+    # 1000, 123, ...) would take the register-staged generic kernels, several times slower; zero columns change
+    # no logit, so e and c are padded once instead (one copy each; autograd cuts the gradients back).
     compute_dtype = _autocast_dtype() or e.dtype
+    if compute_dtype != torch.float32 and e.size(-1) % _D_MULTIPLE != 0:
+        pad = _D_MULTIPLE - e.size(-1) % _D_MULTIPLE
+        e = torch.nn.functional.pad(e, (0, pad))
+        c = torch.nn.functional.pad(c, (0, pad))
+    targets = targets.contiguous()
     filtering = filter_eps is not None
     params = CCEParams(
         targets=targets.flatten(),

@@ -92,6 +92,25 @@ def _target_class(model_type: str):
     return getattr(importlib.import_module(module_name), class_name)
 
 
+def _impl_name(impl) -> str:
+    """Lower-case name of an implementation given as enum member or string; ValueError for an unknown one."""
+    name = impl.name.lower() if isinstance(impl, LinearCrossEntropyImpl) else impl
+    known = {member.name.lower() for member in LinearCrossEntropyImpl}
+    if name not in known:
+        raise ValueError(f"Unknown impl={name!r}")
+    return name
+
+
+def _model_type_of(target) -> str:
+    """The ``model_type`` string of a model, a config, or the string itself; RuntimeError if no patch exists."""
+    if isinstance(target, transformers.PreTrainedModel):
+        target = target.config
+    model_type = target.model_type if isinstance(target, transformers.PretrainedConfig) else target
+    if model_type not in PATCH_TARGETS:
+        raise RuntimeError(f"Unknown model type {model_type}")
+    return model_type
+
+
 def cce_patch(
     model_type_or_model,
     impl: Union[str, LinearCrossEntropyImpl] = LCE_IMPL_DEFAULT,
@@ -106,38 +125,19 @@ def cce_patch(
     """Patch a model instance (returned), or a model family named by type string / config (returns None:
     every instance created afterwards is patched).  ref: transformers/patch.py:53-95.
     """
-    if isinstance(impl, LinearCrossEntropyImpl):
-        impl = impl.name.lower()
-    if impl not in (v.name.lower() for v in LinearCrossEntropyImpl):
-        raise ValueError(f"Unknown {impl=}")
-
-    if isinstance(model_type_or_model, transformers.PreTrainedModel):
-        model_type = model_type_or_model.config.model_type
-    elif isinstance(model_type_or_model, transformers.PretrainedConfig):
-        model_type = model_type_or_model.model_type
-    else:
-        model_type = model_type_or_model
-
-    patch_options = PatchOptions(
-        impl=impl,
-        reduction=reduction,
-        filter_eps=filter_eps,
-        accum_e_fp32=accum_e_fp32,
-        accum_c_fp32=accum_c_fp32,
-        filter_e_grad=filter_e_grad,
-        filter_c_grad=filter_c_grad,
-        train_only=train_only,
-    )
-
-    if model_type not in PATCH_TARGETS:
-        raise RuntimeError(f"Unknown model type {model_type}")
-    cls = _target_class(model_type)
-
-    if isinstance(model_type_or_model, transformers.PreTrainedModel):
-        assert isinstance(model_type_or_model, cls), f"Expected a {cls.__name__} model. Got {type(model_type_or_model)}."
-        setattr(model_type_or_model, _OPTS_ATTR, patch_options)
-        model_type_or_model.forward = MethodType(cce_forward, model_type_or_model)
-        return model_type_or_model
-    setattr(cls, _OPTS_ATTR, patch_options)
+    target = model_type_or_model
+    impl = _impl_name(impl)  # (an unknown impl is reported before an unknown model type, as in the reference)
+    is_instance = isinstance(target, transformers.PreTrainedModel)
+    cls = _target_class(_model_type_of(target))
+    options = PatchOptions(impl=impl, reduction=reduction, filter_eps=filter_eps,
+                           accum_e_fp32=accum_e_fp32, accum_c_fp32=accum_c_fp32,
+                           filter_e_grad=filter_e_grad, filter_c_grad=filter_c_grad, train_only=train_only)
+    if is_instance:
+        # one model: its own bound forward and its own options; other instances of the class stay as they are
+        assert isinstance(target, cls), f"Expected a {cls.__name__} model. Got {type(target)}."
+        setattr(target, _OPTS_ATTR, options)
+        target.forward = MethodType(cce_forward, target)
+        return target
+    setattr(cls, _OPTS_ATTR, options)
     cls.forward = cce_forward
     return None

@@ -52,6 +52,7 @@ def test_host_only_queries():
 
     assert lib.cce_version() == _hip.ABI_VERSION
     assert lib.cce_error_string(0) == b"success"
+    assert lib.cce_source_hash().decode() == _hip._hash_of_sources()  # the library matches the sources beside it
     assert b"workspace" in lib.cce_error_string(10003)
     # ceil(8192 / 32) * ceil(256000 / 32)
     assert lib.cce_tile_stat_elems(8192, 256000) == 256 * 8000
