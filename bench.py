@@ -111,6 +111,21 @@ def loss_fn(w):
     return run
 
 
+def measured_traffic(workload, source_hash):
+    """HBM bytes per launch of the dominant kernel from the committed counter summary, if that summary was
+    taken with the very sources the loaded library is built from (else None: a stale figure is no measurement)."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, "profiles", "lse_forward_c2_hbm_traffic.txt")).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic_bytes=(\S+) workload=(\S+) source_hash=(\S+)", text)
+    if m and m.group(2) == workload and m.group(3) == source_hash:
+        return float(m.group(1)), "profiles/lse_forward_c2_hbm_traffic.txt"
+    return None, None
+
+
 def cpu_baseline(w, rows):
     """Dense oracle (the reference's torch_compile path restated) on the host cores, fp32,
     forward + backward over the first ``rows`` tokens of the same workload."""
@@ -167,7 +182,7 @@ def main():
                     help="also run one plain 1 GiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--traffic", type=float, default=None,
                     help="HBM bytes per launch of the dominant kernel of THIS build, measured with rocprofv3 --pmc; "
-                         "reported as given, null without it")
+                         "reported as given; without it the figure of profiles/ is reported if it belongs to this build")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives); use --gpus 1", file=sys.stderr)
@@ -238,6 +253,10 @@ def main():
     grads = e.grad.numel() * e.grad.element_size() + c.grad.numel() * c.grad.element_size()
     extra_mb = (peak - grads) / 2**20
 
+    traffic, traffic_source = args.traffic, "--traffic" if args.traffic is not None else None
+    if traffic is None:
+        traffic, traffic_source = measured_traffic(w["name"], _hip.load().cce_source_hash().decode())
+
     fwd_ms = kernel_ms["lse_forward"]
     fwd_flops = 2.0 * B * V * D
     fwd_tflops = fwd_flops / (fwd_ms * 1e-3) / 1e12
@@ -279,7 +298,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": fwd_tflops / PEAK_BF16_TFLOPS,
             "ms_per_launch": fwd_ms,
-            "traffic": args.traffic,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
         "backward": {
             "path": bwd_name,
