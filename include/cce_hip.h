@@ -201,8 +201,8 @@ int cce_backward_dz(const void* e, const void* c, const void* bias,
                     float softcap, int dtype, void* stream);
 
 /* Workspace bytes of cce_backward_dense for a dz chunk buffer of at most `max_dz_bytes` (the function rounds
- * it down to whole 256-class tiles of b rows and never goes below one tile), plus the fp32 dE accumulator
- * [b, d] when `d_e_in_workspace` (d_e wanted in the 16-bit input type). */
+ * it down to whole 256-class tiles of b rows, at most 16384 classes, and never goes below one tile), plus the
+ * 16-bit compensation term of dE, [b, d], when `d_e_in_workspace` (d_e wanted in the 16-bit input type). */
 int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace,
                                            int64_t max_dz_bytes);
 
@@ -213,14 +213,16 @@ int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int 
  * the two products d_e += dz . c (:262-275), d_c += dz^T . e (:289-302), which the reference accumulates with
  * atomics.  Here the vocabulary is walked in chunks; per chunk the dz of the chunk is written to the
  * workspace in the input type, d_c[chunk] = dz^T . e and d_bias[chunk] = column sums of dz are complete and
- * written once, and d_e accumulates over the chunks in fp32.
+ * written once, and d_e accumulates over the chunks: in fp32 when d_e is float, else as a pair of 16-bit
+ * numbers, d_e itself and a compensation term in the workspace (the "Kahan" buffers of the reference's
+ * cce_kahan* presets, :374-385: 16 bits of mantissa carried from chunk to chunk, d_e final after the last).
  *
- *   d_e      NULL or [n_rows, d]: float when d_e_is_fp32 (accumulated into: the caller zero-fills), else
- *            `dtype` (rows of valid tokens are written once at the end; other rows are not touched)
+ *   d_e      NULL or [n_rows, d], accumulated into (the caller zero-fills): float when d_e_is_fp32, else `dtype`;
+ *            rows that are not valid tokens are not touched
  *   d_c      NULL or [v, d] with the strides of c; float when d_c_is_fp32 else `dtype`; written, not accumulated
  *   d_bias   NULL or [v] float, accumulated into
  *   workspace  256-byte aligned; at least cce_backward_dense_workspace_bytes(b, v, d, d_e in `dtype`, 0) bytes.
- *            Anything beyond that enlarges the chunks (fewer, better filled launches) up to 8192 classes.
+ *            Anything beyond that enlarges the chunks (fewer, better filled launches) up to 16384 classes.
  * Layout requirements as for cce_backward_dz (16-byte aligned e, c and d_e, unit stride_cd, row strides that
  * are multiples of 8, d a multiple of 64), else CCE_ERR_MISALIGNED and the caller uses cce_backward.
  */

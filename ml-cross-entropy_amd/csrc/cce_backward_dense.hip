@@ -10,8 +10,9 @@
 //   1. dense_dz_kernel    recomputes the logits of the chunk and writes dz [B, vc] in the input type
 //                         (the chunk is sized to stay in the last-level cache),
 //   2. dense_dc_kernel    dC[chunk] = dz^T . E : complete for these classes, written once,
-//   3. dense_de_kernel    dE += dz . C[chunk]  : accumulated in fp32 across the chunks (in d_e itself when the
-//                         caller asked for an fp32 dE, else in the workspace, converted at the end),
+//      (2 and 3 are tiles of one launch, dense_products_kernel)
+//   3. dense_de_kernel    dE += dz . C[chunk]  : accumulated across the chunks in d_e itself, in fp32 when the caller
+//                         asked for an fp32 dE, else as d_e (16 bit) plus a 16-bit compensation term in the workspace,
 //   4. dz_colsum_kernel   dBias[chunk], when wanted.
 // Both products run on the tile loop of cce_tile4.h (direct-to-LDS loads, LDS transpose reads for the
 // operand whose reduction index is the row index).  Everything is enqueued on the caller's stream; nothing
@@ -32,9 +33,11 @@ struct ProductParams {
   const uint16_t* e;
   int64_t stride_e;
   const int32_t* valids;
-  float* de_acc;        // fp32 accumulator of dE
-  int64_t ld_acc;
-  int acc_by_valids;    // rows of de_acc are rows of e (through valids) rather than valid-row numbers
+  float* de_f32;        // dE accumulated in fp32, in the caller's float d_e (rows of e, through valids); or nullptr:
+  uint16_t* de_hi;      // dE accumulated as a pair of 16-bit values hi + lo: hi is the caller's d_e in the input type
+  uint16_t* de_lo;      //   (rows of e), lo the compensation term in the workspace ([b][d], rows by valid-row number)
+  int64_t ld_de;        // row stride of d_e (elements)
+  int first_chunk;      // nothing accumulated yet: the pair is written, not read
   void* d_c;            // first class of the chunk
   int dc_fp32;
   int64_t b;
@@ -59,7 +62,7 @@ __device__ __forceinline__ bool product_tile_of(int block, int tiles, int per_xc
 }
 
 // dE[row][col] += sum_class dz[row][class] * C[class][col]
-template <typename T>
+template <typename T, bool SPLIT_DE>
 __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, int tn, unsigned char* smem) {
   using Tile = Tile4<T, false, true>;
   typename Tile::Geometry g = Tile::geometry(smem);
@@ -91,30 +94,46 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
   Tile::prefetch(s, ptrs, ids, g);
   Tile::run(acc, s, ptrs, ids, smem, g);
 
-#pragma unroll
-  for (int j = 0; j < Tile::WN; ++j) {
-    const int col = n0 + g.wn * 128 + j * 32 + g.l32;
-    if (col >= p.d) continue;
-#pragma unroll
-    for (int i = 0; i < Tile::WM; ++i) {
-      float* dst[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t row_i = m0 + g.wm * 128 + i * 32 + 8 * (r >> 2) + 4 * g.half + (r & 3);
-        dst[r] = nullptr;
-        if (row_i < p.b) {
-          const int64_t row = (p.acc_by_valids && p.valids != nullptr) ? static_cast<int64_t>(p.valids[row_i]) : row_i;
-          dst[r] = p.de_acc + row * p.ld_acc + col;
-        }
+  Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
+    const int64_t ri = m0 + row;          // valid-row number
+    const int cg = n0 + col;
+    if (ri >= p.b || cg >= p.d) return;
+    const int64_t re = (p.valids != nullptr) ? static_cast<int64_t>(p.valids[ri]) : ri;  // its row of e
+    if (!SPLIT_DE) {
+      float4* dst = reinterpret_cast<float4*>(p.de_f32 + re * p.ld_de + cg);
+      float4 a = dst[0], b = dst[1];
+      a.x += v[0]; a.y += v[1]; a.z += v[2]; a.w += v[3];
+      b.x += v[4]; b.y += v[5]; b.z += v[6]; b.w += v[7];
+      dst[0] = a;
+      dst[1] = b;
+    } else {
+      // value so far = hi + lo (two 16-bit numbers: 16 bits of mantissa, where one would round the sum of a few
+      // dozen chunks eight bits short); the new hi is the rounded total, so the last chunk leaves d_e final
+      uint4* hi_ptr = reinterpret_cast<uint4*>(p.de_hi + re * p.ld_de + cg);
+      uint4* lo_ptr = reinterpret_cast<uint4*>(p.de_lo + ri * p.d + cg);
+      uint4 hi = make_uint4(0u, 0u, 0u, 0u), lo = make_uint4(0u, 0u, 0u, 0u);
+      if (!p.first_chunk) {
+        hi = *hi_ptr;
+        lo = *lo_ptr;
       }
-      float old[16];
+      const uint32_t hw[4] = {hi.x, hi.y, hi.z, hi.w}, lw[4] = {lo.x, lo.y, lo.z, lo.w};
+      uint32_t ho[4], lo_out[4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) old[r] = (dst[r] != nullptr) ? *dst[r] : 0.0f;
+      for (int k = 0; k < 4; ++k) {
+        float t[2], rest[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (dst[r] != nullptr) *dst[r] = old[r] + acc[i][j][r];
+        for (int h = 0; h < 2; ++h)
+          t[h] = (Elem<T>::to_float(static_cast<uint16_t>(hw[k] >> (16 * h))) +
+                  Elem<T>::to_float(static_cast<uint16_t>(lw[k] >> (16 * h)))) + v[2 * k + h];
+        ho[k] = Elem<T>::pack2(t[0], t[1]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) rest[h] = t[h] - Elem<T>::to_float(static_cast<uint16_t>(ho[k] >> (16 * h)));
+        lo_out[k] = Elem<T>::pack2(rest[0], rest[1]);
+      }
+      *hi_ptr = make_uint4(ho[0], ho[1], ho[2], ho[3]);
+      *lo_ptr = make_uint4(lo_out[0], lo_out[1], lo_out[2], lo_out[3]);
     }
-  }
+  });
 }
 
 // dC[class][col] = sum_row dz[row][class] * E[row][col]
@@ -145,29 +164,26 @@ __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, in
   Tile::prefetch(s, ptrs, ids, g);
   Tile::run(acc, s, ptrs, ids, smem, g);
 
-#pragma unroll
-  for (int j = 0; j < Tile::WN; ++j) {
-    const int col = n0 + g.wn * 128 + j * 32 + g.l32;
-    if (col >= p.d) continue;
-#pragma unroll
-    for (int i = 0; i < Tile::WM; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int cls = m0 + g.wm * 128 + i * 32 + 8 * (r >> 2) + 4 * g.half + (r & 3);
-        if (cls < p.n_cls) {
-          const int64_t off = static_cast<int64_t>(cls) * p.stride_cv + col;
-          if (p.dc_fp32) static_cast<float*>(p.d_c)[off] = acc[i][j][r];
-          else static_cast<uint16_t*>(p.d_c)[off] = Elem<T>::from_float(acc[i][j][r]);
-        }
-      }
+  Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
+    const int cls = m0 + row;
+    const int cg = n0 + col;
+    if (cls >= p.n_cls || cg >= p.d) return;
+    const int64_t off = static_cast<int64_t>(cls) * p.stride_cv + cg;
+    if (p.dc_fp32) {
+      float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.d_c) + off);
+      dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+      dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+      *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.d_c) + off) =
+          make_uint4(Elem<T>::pack2(v[0], v[1]), Elem<T>::pack2(v[2], v[3]), Elem<T>::pack2(v[4], v[5]), Elem<T>::pack2(v[6], v[7]));
     }
-  }
+  });
 }
 
 // Both products of one chunk in one launch: the dC tiles (reduction over all B rows) take the first block ids,
 // the dE tiles (reduction over the classes of the chunk) the rest.  Blocks are handed to compute units in id
 // order as units fall free, so the two kinds fill each other's last round.
-template <typename T>
+template <typename T, bool SPLIT_DE>
 __global__ __launch_bounds__(kProdThreads, 1) void dense_products_kernel(ProductParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int dc_blocks = p.dc_per_xcd * 8;
@@ -177,7 +193,7 @@ __global__ __launch_bounds__(kProdThreads, 1) void dense_products_kernel(Product
     dense_dc_tile<T>(p, tm, tn, smem);
   } else {
     if (!product_tile_of(blockIdx.x - dc_blocks, p.de_tiles, p.de_per_xcd, p.tiles_n, tm, tn)) return;
-    dense_de_tile<T>(p, tm, tn, smem);
+    dense_de_tile<T, SPLIT_DE>(p, tm, tn, smem);
   }
 }
 
@@ -200,30 +216,6 @@ __global__ __launch_bounds__(1024) void dz_colsum_kernel(const uint16_t* dz, int
     for (int j = 0; j < 16; ++j) t += part[j][cl];  // fixed order: deterministic
     d_bias[cls] += t;
   }
-}
-
-__global__ void dense_fill_zero_kernel(float4* p, int64_t n4) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < n4) p[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-}
-
-// d_e[row of valid row i][:] = round(acc[i][:]), eight columns per thread
-template <typename T>
-__global__ void dense_store_de_kernel(const float* acc, const int32_t* valids, uint16_t* d_e, int64_t stride_e, int64_t b,
-                                      int d8) {
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= b * d8) return;
-  const int64_t i = idx / d8;
-  const int c8 = static_cast<int>(idx - i * d8);
-  const float4 lo = *reinterpret_cast<const float4*>(acc + (i * d8 + c8) * 8);
-  const float4 hi = *reinterpret_cast<const float4*>(acc + (i * d8 + c8) * 8 + 4);
-  uint4 out;
-  out.x = Elem<T>::pack2(lo.x, lo.y);
-  out.y = Elem<T>::pack2(lo.z, lo.w);
-  out.z = Elem<T>::pack2(hi.x, hi.y);
-  out.w = Elem<T>::pack2(hi.z, hi.w);
-  const int64_t row = valids ? static_cast<int64_t>(valids[i]) : i;
-  *reinterpret_cast<uint4*>(d_e + row * stride_e + c8 * 8) = out;
 }
 
 static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de,
@@ -276,7 +268,7 @@ static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int
                                             bool want_dc) {
   const int64_t v_pad = (v + 255) / 256 * 256;
   int64_t top = max_dz_bytes / (b * 2) / 256 * 256;
-  if (top > 8192) top = 8192;
+  if (top > 16384) top = 16384;
   if (top < 256) return 0;
   if (top >= v_pad) return v_pad;
   const int64_t col_tiles = (d + 255) / 256;
@@ -315,8 +307,8 @@ extern "C" int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int6
   if (b <= 0 || v <= 0 || d <= 0) return 0;
   int64_t vc = dense_chunk_classes(b, v, d, max_dz_bytes, true, true);
   if (vc == 0) vc = 256;  // the smallest plan
-  const int64_t acc = d_e_in_workspace ? align256(b * d * 4) : 0;
-  return acc + align256(b * vc * 2);
+  const int64_t comp = d_e_in_workspace ? align256(b * d * 2) : 0;  // the compensation half of dE
+  return comp + align256(b * vc * 2);
 }
 
 extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias,
@@ -342,25 +334,18 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   if (!aligned16(e) || !aligned16(c) || d % kDmaBK != 0 || stride_e % 8 != 0 || stride_cv % 8 != 0 || stride_cd != 1)
     return CCE_ERR_MISALIGNED;
   if (stride_e >= (int64_t(1) << 30) || stride_cv >= (int64_t(1) << 30)) return CCE_ERR_INVALID_ARGUMENT;
-  if (d_e != nullptr && !aligned16(d_e)) return CCE_ERR_MISALIGNED;
+  if ((d_e != nullptr && !aligned16(d_e)) || (d_c != nullptr && !aligned16(d_c))) return CCE_ERR_MISALIGNED;
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
     return workspace == nullptr ? CCE_ERR_WORKSPACE_TOO_SMALL : CCE_ERR_MISALIGNED;
 
-  // ---- plan: [fp32 dE accumulator][dz chunk] -------------------------------------------------------------
-  const bool acc_in_ws = (d_e != nullptr) && !d_e_is_fp32;
-  const int64_t acc_bytes = acc_in_ws ? align256(b * d * 4) : 0;
+  // ---- plan: [16-bit compensation term of dE][dz chunk] ----------------------------------------------------
+  const bool split_de = (d_e != nullptr) && !d_e_is_fp32;
+  const int64_t comp_bytes = split_de ? align256(b * d * 2) : 0;
   // the plan the size query made (both gradients wanted), so that its answer always suffices
-  const int64_t vc = dense_chunk_classes(b, v, d, workspace_bytes - acc_bytes, true, true);
+  const int64_t vc = dense_chunk_classes(b, v, d, workspace_bytes - comp_bytes, true, true);
   if (vc == 0) return CCE_ERR_WORKSPACE_TOO_SMALL;
-  float* acc = acc_in_ws ? static_cast<float*>(workspace) : static_cast<float*>(d_e);
-  uint16_t* dz = reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + acc_bytes);
+  uint16_t* dz = reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + comp_bytes);
   const int64_t ldz = vc;
-
-  if (acc_in_ws) {
-    const int64_t n4 = b * d / 4;
-    hipLaunchKernelGGL(dense_fill_zero_kernel, dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0, stream,
-                       reinterpret_cast<float4*>(acc), n4);
-  }
 
   ProductParams p;
   p.dz = dz;
@@ -369,9 +354,10 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   p.e = static_cast<const uint16_t*>(e);
   p.stride_e = stride_e;
   p.valids = valids;
-  p.de_acc = acc;
-  p.ld_acc = acc_in_ws ? d : stride_e;
-  p.acc_by_valids = acc_in_ws ? 0 : 1;
+  p.de_f32 = split_de ? nullptr : static_cast<float*>(d_e);
+  p.de_hi = split_de ? static_cast<uint16_t*>(d_e) : nullptr;
+  p.de_lo = split_de ? static_cast<uint16_t*>(workspace) : nullptr;
+  p.ld_de = stride_e;
   p.dc_fp32 = d_c_is_fp32;
   p.b = b;
   p.d = static_cast<int>(d);
@@ -400,6 +386,7 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
     if (st != CCE_OK) return st;
     p.c = reinterpret_cast<const uint16_t*>(c_chunk);
     p.n_cls = static_cast<int>(n);
+    p.first_chunk = (v0 == 0) ? 1 : 0;
     p.tiles_n = tiles_n;
     p.d_c = nullptr;
     p.dc_tiles = 0;
@@ -412,8 +399,13 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
     p.de_per_xcd = (p.de_tiles + 7) / 8;
     const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
     if (blocks > 0) {
-      if (dtype == CCE_DTYPE_BF16) CCE_LAUNCH_PRODUCT(dense_products_kernel<BF16>, blocks);
-      else CCE_LAUNCH_PRODUCT(dense_products_kernel<F16>, blocks);
+      if (dtype == CCE_DTYPE_BF16) {
+        if (split_de) CCE_LAUNCH_PRODUCT((dense_products_kernel<BF16, true>), blocks);
+        else CCE_LAUNCH_PRODUCT((dense_products_kernel<BF16, false>), blocks);
+      } else {
+        if (split_de) CCE_LAUNCH_PRODUCT((dense_products_kernel<F16, true>), blocks);
+        else CCE_LAUNCH_PRODUCT((dense_products_kernel<F16, false>), blocks);
+      }
     }
     if (d_bias != nullptr) {
       const unsigned blocks = static_cast<unsigned>((n + 63) / 64);
@@ -429,16 +421,5 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   }
 #undef CCE_LAUNCH_PRODUCT
 
-  if (acc_in_ws) {
-    const int d8 = static_cast<int>(d / 8);
-    const int64_t total = b * d8;
-    const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
-    if (dtype == CCE_DTYPE_BF16)
-      hipLaunchKernelGGL(dense_store_de_kernel<BF16>, dim3(blocks), dim3(256), 0, stream, acc, valids,
-                         static_cast<uint16_t*>(d_e), stride_e, b, d8);
-    else
-      hipLaunchKernelGGL(dense_store_de_kernel<F16>, dim3(blocks), dim3(256), 0, stream, acc, valids,
-                         static_cast<uint16_t*>(d_e), stride_e, b, d8);
-  }
   return status_from_hip(hipGetLastError());
 }

@@ -26,6 +26,8 @@
 // cannot see them.
 #pragma once
 
+#include <utility>
+
 #include "cce_common.h"
 
 namespace cce {
@@ -33,6 +35,17 @@ namespace cce {
 static __device__ __align__(256) uint16_t g_zero_line[128];  // never written
 
 typedef short tr_short4_t __attribute__((ext_vector_type(4)));
+
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
+// in every iteration, whatever the size of its body (an array of accumulators indexed by it stays in registers).
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <typename T, bool A_KM, bool B_KM>
 struct Tile4 {
@@ -360,6 +373,46 @@ struct Tile4 {
     if (nk & 1) stage<0>(acc, fa, fb, lds, s, nk - 1, ptrs, ids, g);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch
     __syncthreads();
+  }
+
+  // ---- the finished tile, as row pieces ----------------------------------------------------------------
+  // The accumulators hold the tile with its columns along the lanes: written out as they are, a lane would
+  // touch one element (2 or 4 bytes) of 16 rows.  Each wave instead passes its 128 x 128 part through LDS (idle
+  // after run()), 32 rows x 64 columns at a time, and hands `f` pieces of 8 consecutive columns of one row:
+  //     f(row, col, v)   row, col: position inside the 256 x 256 tile; v[8]: the values [row][col .. col + 7]
+  // so that a piece is one 16-byte (16-bit data) or two 16-byte (fp32) accesses and 8 lanes cover 128 or 256
+  // contiguous bytes of a row.  The staging area is private to the wave: no barrier.
+  static constexpr int kPieceCols = 8;
+  static constexpr int kStagePitch = (64 + 4) * 4;           // bytes per staged row
+  static constexpr int kStageBytes = 32 * kStagePitch;       // per wave
+  static_assert(NW * kStageBytes <= LDS_BYTES, "the staging areas reuse the ring");
+
+  template <typename F>
+  static __device__ __forceinline__ void for_each_row_piece(f32x16 (&acc)[WM][WN], unsigned char* lds, const Geometry& g,
+                                                            F&& f) {
+    unsigned char* stage = lds + g.wave * kStageBytes;
+    static_for<WM * (WN / 2)>([&](auto ij) {
+      constexpr int i = decltype(ij)::value / (WN / 2);
+      constexpr int jp = decltype(ij)::value % (WN / 2);
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = 8 * (r >> 2) + 4 * g.half + (r & 3);
+          *reinterpret_cast<float*>(stage + m * kStagePitch + (jj * 32 + g.l32) * 4) = acc[i][jp * 2 + jj][r];
+        }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int pass = 0; pass < 4; ++pass) {
+        const int m = pass * 8 + (g.lane >> 3);
+        const int c8 = (g.lane & 7) * kPieceCols;
+        const float4 lo = *reinterpret_cast<const float4*>(stage + m * kStagePitch + c8 * 4);
+        const float4 hi = *reinterpret_cast<const float4*>(stage + m * kStagePitch + c8 * 4 + 16);
+        const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        f(g.wm * 128 + i * 32 + m, g.wn * 128 + jp * 64 + c8, v);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the next slab is staged
+    });
   }
 };
 
