@@ -620,7 +620,7 @@ constexpr int kFStageBytes = kFOtherBytes + kFOwnBytes;
 constexpr int kFMaxChunks = 18;                     // 18 * 128 = 2304 columns of D per workgroup
 constexpr int kFOffDz = 3 * kFStageBytes;           // 120 KB
 constexpr int kFOffList = kFOffDz + 8 * 1024;       //   8 KB entry list (2048 entries)
-constexpr int kFOffFlag = kFOffList + 8 * 1024;     // 512 B
+constexpr int kFOffFlag = kFOffList + 8 * 1024 + 16; // 512 B (the list holds 2048 entries + 3 carried over)
 constexpr int kFOffBits = kFOffFlag + 512;          //   8 KB
 constexpr int kFOffMeta = kFOffBits + kMaxBitWords * 4;
 constexpr int kFLdsBytes = kFOffMeta + 5 * kMetaRows * 4 + 32 * 4 + 128 * 4 + 128 * 4 + 64;
@@ -757,6 +757,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
   const int n_units = IS_DE ? p.nvc : p.ntg;
   const int seg_units = IS_DE ? kFSegCells : kFListCap;
 
+  int carry = 0;  // listed entries a segment left over for the next one (trips are filled four at a time)
   for (int seg = 0; seg < n_units; seg += seg_units) {
     const int seg_n = min(seg_units, n_units - seg);
     if (use_list) {
@@ -783,7 +784,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         __syncthreads();
       }
       if (wave == 0) {
-        int n = 0;
+        int n = carry;
         uint32_t kept_word[4] = {0u, 0u, 0u, 0u};
         for (int base = 0; base < seg_n; base += 64) {
           if (IS_DE) {
@@ -823,9 +824,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
     }
     const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
     // A class group nothing survived for: its rows keep the zeros they came with.
-    if (!IS_DE && list_n == 0 && n_units <= seg_units) return;
+    if (!IS_DE && list_n == 0 && n_units <= seg_units) break;
+    // Only the last segment runs a trip that is not full: what is left over goes to the front of the next list.
+    const bool keep_rest = use_list && (seg + seg_units < n_units);
+    const int run_n = keep_rest ? (list_n & ~3) : list_n;
 
-    for (int li = 0; li < list_n; li += 4) {
+    for (int li = 0; li < run_n; li += 4) {
       if (IS_DE) {
         if (tid < 128) {
           const int k = li + (tid >> 5);
@@ -877,48 +881,115 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       const int slot_bytes = own_off + kFOwnBytes;
       const int ring = (nent >= 3) ? 3 : ((nent == 2) ? 5 : 7);  // slots of this size in the 120 KB ring
       const int ahead = ring - 1;                              // stages in flight
-      auto issue_stage = [&](int col0, int slot, bool with_own, uint32_t entries) {
+      // load q of this wave for the stage that starts at column col0: q < 8 other side, q = 8, 9 own side
+      auto issue_load = [&](int q, int col0, int slot, bool with_own, uint32_t entries) {
         const unsigned base = lds_base + slot * slot_bytes;
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
+        if (q < 8) {
           if ((entries >> (q >> 1)) & 1u)
-            lds_dma16(other_ptr[q] + (((other_live >> q) & 1u) ? col0 : 0), base + (q * 4 + wave) * 1024);
-        if (with_own) {
-#pragma unroll
-          for (int q = 0; q < 2; ++q) lds_dma16(own_ptr[q] + (own_step[q] ? col0 : 0), base + own_off + (q * 4 + wave) * 1024);
+            lds_dma16(other_ptr[q & 7] + (((other_live >> q) & 1u) ? col0 : 0), base + (q * 4 + wave) * 1024);
+        } else if (with_own) {
+          lds_dma16(own_ptr[q & 1] + (own_step[q & 1] ? col0 : 0), base + own_off + ((q - 8) * 4 + wave) * 1024);
         }
+      };
+      auto issue_stage = [&](int col0, int slot, bool with_own, uint32_t entries) {
+#pragma unroll
+        for (int q = 0; q < 10; ++q) issue_load(q, col0, slot, with_own, entries);
       };
 
       // ---- logits^T of (entry of this wave) x (own rows): 2 nent + 2 loads per wave and stage -----------
+      // One wave per SIMD issues every instruction of this loop by itself, so the loop is written once per
+      // number of entries: ring geometry, wait counts and which loads exist are then compile-time facts and
+      // the body is straight-line code.
       f32x16 s;
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-      const int last_col = (nstages - 1) * kFCols;
-      const uint32_t present = (1u << nent) - 1u;
+      auto logits_of_trip = [&](auto nent_tag) {
+        constexpr int NENT = decltype(nent_tag)::value;
+        constexpr int KPARTS = (NENT == 1) ? 4 : ((NENT == 2) ? 2 : 1);
+        constexpr int NKK = 8 / KPARTS;
+        constexpr int OWN_OFF = 32 * NENT * kFRowBytes;
+        constexpr int SLOT = OWN_OFF + kFOwnBytes;
+        constexpr int RING = (NENT >= 3) ? 3 : ((NENT == 2) ? 5 : 7);
+        constexpr int AHEAD = RING - 1;
+        constexpr int PER_STAGE = 2 * NENT + 2;
+        auto issue = [&](auto q_tag, int col0, unsigned base) {
+          constexpr int Q = decltype(q_tag)::value;
+          if constexpr (Q < 2 * NENT) {
+            lds_dma16(other_ptr[Q] + (((other_live >> Q) & 1u) ? col0 : 0), base + (Q * 4 + wave) * 1024);
+          } else if constexpr (Q >= 8) {
+            lds_dma16(own_ptr[Q - 8] + (own_step[Q - 8] ? col0 : 0), base + OWN_OFF + ((Q - 8) * 4 + wave) * 1024);
+          }
+        };
+        // the MFMAs of stage `slot`; with ISSUE the loads of column block next_col go out among them
+        auto step = [&](auto issue_tag, int slot, int next_col, int next_slot) {
+          constexpr bool ISSUE = decltype(issue_tag)::value;
+          const unsigned char* so = smem + slot * SLOT;
+          const unsigned char* sw = so + OWN_OFF;
+          const unsigned nbase = lds_base + next_slot * SLOT;
+          // All fragment reads of a half stage go out first, then loads (their issue is what takes longest in a
+          // step: the reads land meanwhile) with the MFMAs in between.
+          typename Elem<T>::vec8 fo[4], fw[4];
+          auto read_half = [&](int j0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              if (j0 + j < NKK) {
+                const int kk = kpart * NKK + j0 + j;
+                fo[j] = fstage_frag<T>(so, ew * 32 + l32, kk * 2 + half);
+                fw[j] = fstage_frag<T>(sw, l32, kk * 2 + half);
+              }
+            }
+          };
+          auto mfma_of = [&](int j) {
+            if (IS_DE) Elem<T>::mfma_vgpr(fo[j], fw[j], s);
+            else Elem<T>::mfma_vgpr(fw[j], fo[j], s);
+          };
+          read_half(0);
+          if constexpr (ISSUE) {
+            issue(std::integral_constant<int, 0>{}, next_col, nbase);
+            issue(std::integral_constant<int, 1>{}, next_col, nbase);
+          }
+          static_for<4>([&](auto j) {
+            if constexpr (j.value < NKK) mfma_of(j.value);
+            if constexpr (ISSUE) issue(std::integral_constant<int, 2 + j.value>{}, next_col, nbase);
+          });
+          if constexpr (NKK == 8) read_half(4);
+          if constexpr (ISSUE) {
+            issue(std::integral_constant<int, 6>{}, next_col, nbase);
+            issue(std::integral_constant<int, 7>{}, next_col, nbase);
+          }
+          static_for<4>([&](auto j) {
+            if constexpr (NKK == 8) mfma_of(j.value);
+            if constexpr (ISSUE && j.value < 2) issue(std::integral_constant<int, 8 + j.value>{}, next_col, nbase);
+          });
+        };
+
+        const int npre = min(AHEAD, nstages);
 #pragma unroll 1
-      for (int j = 0; j < ahead; ++j) issue_stage(min(j * kFCols, last_col), j, true, present);
-      int slot = 0;  // st % ring
+        for (int j = 0; j < npre; ++j)
+          static_for<10>([&](auto q) { issue(q, j * kFCols, lds_base + j * SLOT); });
+        int slot = 0;  // st % RING
+        const int nsteady = nstages - npre;  // steps that still have a stage to start
 #pragma unroll 1
-      for (int st = 0; st < nstages; ++st) {
-        wait_vmcnt_upto((ahead - 1) * (2 * nent + 2));  // all but the newest stages have landed
-        __syncthreads();                                   // ... for every wave; stage st - 1 is consumed
-        issue_stage(min((st + ahead) * kFCols, last_col), (slot == 0) ? ring - 1 : slot - 1, true, present);
-        const unsigned char* so = smem + slot * slot_bytes;
-        const unsigned char* sw = so + own_off;
-        slot = (slot + 1 == ring) ? 0 : slot + 1;
-        const int nkk = 8 / kparts;
-#pragma unroll 2
-        for (int j = 0; j < nkk; ++j) {
-          const int kk = kpart * nkk + j;
-          const auto fo = fstage_frag<T>(so, ew * 32 + l32, kk * 2 + half);
-          const auto fw = fstage_frag<T>(sw, l32, kk * 2 + half);
-          if (IS_DE) Elem<T>::mfma_vgpr(fo, fw, s);
-          else Elem<T>::mfma_vgpr(fw, fo, s);
+        for (int st = 0; st < nsteady; ++st) {
+          wait_vmcnt<(AHEAD - 1) * PER_STAGE>();  // all but the newest stages have landed
+          __syncthreads();                          // ... for every wave; stage st - 1 is consumed
+          const int next_slot = (slot == 0) ? RING - 1 : slot - 1;
+          step(std::true_type{}, slot, (st + AHEAD) * kFCols, next_slot);
+          slot = (slot + 1 == RING) ? 0 : slot + 1;
         }
-      }
+#pragma unroll 1
+        for (int st = nsteady; st < nstages; ++st) {
+          wait_vmcnt_upto((nstages - 1 - st) * PER_STAGE);
+          __syncthreads();
+          step(std::false_type{}, slot, 0, 0);
+          slot = (slot + 1 == RING) ? 0 : slot + 1;
+        }
+      };
+      if (nent >= 3) logits_of_trip(std::integral_constant<int, 4>{});
+      else if (nent == 2) logits_of_trip(std::integral_constant<int, 2>{});
+      else logits_of_trip(std::integral_constant<int, 1>{});
       mfma_drain(s);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the unused prefetches
-      __syncthreads();
+      __syncthreads();  // every load has landed and every stage is consumed
       if (kparts > 1) {  // partial logits -> the owner, through the idle ring, in a fixed order
         float* sRed = reinterpret_cast<float*>(smem);
         if (!owner) {
@@ -934,7 +1005,6 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         }
         __syncthreads();  // before the product phase refills the ring
       }
-      const int last_chunk_col = d_begin + (nchunks - 1) * kFCols;
 
       // ---- dz of the owner's 32 x 32 block (lane = token row, registers = classes) ----------------------------
       if (owner) {
@@ -995,23 +1065,35 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       if (product) {
         // Only the entries that are used are fetched again: the others would be read for nothing.
         const int nused = __popc(mask);
+        const int npre = min(ahead, nchunks);
 #pragma unroll 1
-        for (int j = 0; j < ahead; ++j) issue_stage(min(d_begin + j * kFCols, last_chunk_col), j, false, mask);
+        for (int j = 0; j < npre; ++j) issue_stage(d_begin + j * kFCols, j, false, mask);
         int pslot = 0;  // ci % ring
 #pragma unroll
         for (int ci = 0; ci < kFMaxChunks; ++ci) {
           if (ci < nchunks) {
-            wait_vmcnt_upto((ahead - 1) * 2 * nused);
+            wait_vmcnt_upto(min(ahead - 1, nchunks - 1 - ci) * 2 * nused);  // the stages after ci may be in flight
             __syncthreads();
-            issue_stage(min(d_begin + (ci + ahead) * kFCols, last_chunk_col), (pslot == 0) ? ring - 1 : pslot - 1, false, mask);
             const unsigned char* so = smem + pslot * slot_bytes;
+            const int next_col = d_begin + (ci + ahead) * kFCols;
+            const uint32_t next_mask = (ci + ahead < nchunks) ? mask : 0u;  // nothing is fetched past the slice
+            const int next_slot = (pslot == 0) ? ring - 1 : pslot - 1;
             pslot = (pslot + 1 == ring) ? 0 : pslot + 1;
+            // as in the logit phase: reads, then loads with the MFMAs in between
+            typename Elem<T>::vec8 a[4];
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) {
-              if ((mask >> (kk >> 1)) & 1u) {
-                const auto a = fstage_frag_transposed<T>(so, kk * 16, wave * 32, lane);
-                if (ci < 16) Elem<T>::mfma_agpr(a, bz[kk], acc[ci]);  // 16 chunks fill the 256 AGPRs
-                else Elem<T>::mfma_vgpr(a, bz[kk], acc[ci]);
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if ((mask >> ((4 * h + j) >> 1)) & 1u) a[j] = fstage_frag_transposed<T>(so, (4 * h + j) * 16, wave * 32, lane);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int kk = 4 * h + j;
+                issue_load(kk, next_col, next_slot, false, next_mask);
+                if ((mask >> (kk >> 1)) & 1u) {
+                  if (ci < 16) Elem<T>::mfma_agpr(a[j], bz[kk], acc[ci]);  // 16 chunks fill the 256 AGPRs
+                  else Elem<T>::mfma_vgpr(a[j], bz[kk], acc[ci]);
+                }
               }
             }
           }
@@ -1019,6 +1101,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain before the ring is refilled
       __syncthreads();
+    }
+    carry = keep_rest ? list_n - run_n : 0;
+    if (tid < carry) {  // wave 0, which also builds the next list: LDS operations of one wave stay in order
+      const int rest = sList[run_n + tid];
+      sList[tid] = rest;
     }
   }
 

@@ -9,6 +9,8 @@
 // statistics a register-local reduction.
 #pragma once
 
+#include <utility>
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -298,6 +300,23 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, unsigned lds_addr) {
                : "memory", "m0");
 }
 #pragma clang diagnostic pop
+
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
+// in every iteration, whatever the size of its body (an array of accumulators indexed by it stays in registers).
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// s_waitcnt vmcnt(N) with a compile-time N
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 constexpr int kDmaBK = 64;
 constexpr int kDmaRowBytes = 128;

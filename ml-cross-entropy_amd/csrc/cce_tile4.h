@@ -36,17 +36,6 @@ static __device__ __align__(256) uint16_t g_zero_line[128];  // never written
 
 typedef short tr_short4_t __attribute__((ext_vector_type(4)));
 
-template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
-// in every iteration, whatever the size of its body (an array of accumulators indexed by it stays in registers).
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 template <typename T, bool A_KM, bool B_KM>
 struct Tile4 {
   static constexpr int WM = 4, WN = 4;   // accumulator blocks per wave
