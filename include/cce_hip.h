@@ -143,7 +143,8 @@ int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d);
  *   tile_max   NULL or the statistic written by cce_lse_forward for the same inputs
  *   d_e        NULL or [n_rows, d] accumulated into (caller zero-fills); float when
  *              d_e_is_fp32 else `dtype`; same strides as e
- *   d_c        NULL or [v, d]; float when d_c_is_fp32 else `dtype`; same strides as c
+ *   d_c        NULL or [v, d], written: every element when b > 0 (zeros where no tile survived), nothing
+ *              when b == 0; need not be initialised; float when d_c_is_fp32 else `dtype`; same strides as c
  *   d_bias     NULL or [v] float, accumulated into
  *   counters   NULL or CCE_NUM_COUNTERS uint64, accumulated into
  */

@@ -549,8 +549,9 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_kernel(BwdParams p) 
     }
   }
 
-  // ---- write the own rows once; rows nobody touched keep the caller's zeros ------------------------------
-  if (write_out && touched) {
+  // ---- write the own rows once: a row group nobody touched keeps the zeros dE came with; a class group
+  // always writes its rows of dC (zeros when nothing survived for it), so dC need not be cleared beforehand
+  if (write_out && (touched || !IS_DE)) {
     const int id = own_ids[l32];
     if (id >= 0) {
 #pragma unroll
@@ -823,7 +824,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       __syncthreads();
     }
     const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
-    // A class group nothing survived for: its rows keep the zeros they came with.
+    // A class group nothing survived for goes straight to writing its zeros.
     if (!IS_DE && list_n == 0 && n_units <= seg_units) break;
     // Only the last segment runs a trip that is not full: what is left over goes to the front of the next list.
     const bool keep_rest = use_list && (seg + seg_units < n_units);
@@ -1111,7 +1112,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 
   mfma_drain_all();  // the last product MFMAs, before anything else reads the accumulators
   const bool out_fp32 = IS_DE ? (p.de_fp32 != 0) : (p.dc_fp32 != 0);
-  if (write_out && touched) {  // the launcher guarantees 16-byte aligned output rows
+  if (write_out && (touched || !IS_DE)) {  // dC rows are always written; the launcher guarantees 16-byte aligned rows
     // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
     // are, one instruction would touch 32 rows with 16 bytes each.  Four chunks at a time go through
     // LDS instead and leave as whole rows, 16 bytes per lane and 1 KB per row and instruction.

@@ -213,19 +213,24 @@ def cce_backward_kernel(
         # the products of the dense path accumulate in fp32 registers and each output element is written once
         # (dC, dBias) or summed over the chunks in an fp32 workspace (dE): no fp32 gradient buffers are needed
         de_dtype, dc_dtype = e_info.dtype, c_info.dtype
+    n_valid_rows = valids.size(0) if valids is not None else e.size(0)
     de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
     dc = None
     if c_info.requires_grad:
-        # the dense path writes every element of dC; the ownership kernels leave untouched rows to the zeros
-        dc = torch.empty_like(c, dtype=dc_dtype) if dense else torch.zeros_like(c, dtype=dc_dtype)
+        # both paths write every element of dC (the ownership kernel stores zeros for a class group nothing
+        # survived for); only with no valid row at all is nothing launched
+        dc = torch.empty_like(c, dtype=dc_dtype) if n_valid_rows > 0 else torch.zeros_like(c, dtype=dc_dtype)
         if dc.stride() != c.stride():
-            # a view with gaps between its rows or columns (zeros_like packs those): the kernels address C and
+            # a view with gaps between its rows or columns (empty_like packs those): the kernels address C and
             # dC with one pair of strides, so dC gets the layout of c, or c is packed if its elements overlap
             (s_small, n_small), (s_large, _) = sorted(zip(c.stride(), c.size()))
             if s_small >= 1 and s_large >= s_small * n_small:
-                dc = torch.empty_strided(c.size(), c.stride(), dtype=dc_dtype, device=dev).zero_()
+                dc = torch.empty_strided(c.size(), c.stride(), dtype=dc_dtype, device=dev)
+                if n_valid_rows == 0:
+                    dc.zero_()
             else:
                 c = c.contiguous()
+                dc = dc.contiguous()
     dbias = None
     if bias is not None:
         assert bias_info is not None

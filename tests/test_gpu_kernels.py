@@ -109,7 +109,8 @@ def _run_backward_abi(e, c, t, bias, valids, lse, d_out, d_lse, softcap, shift, 
     od = order.to(dev) if order is not None else None
     gdt = torch.float32 if fp32_accum else dtype
     de = torch.zeros((N, D), dtype=gdt, device=dev)
-    dc = torch.zeros((V, D), dtype=gdt, device=dev)
+    # d_c need not be initialised: the kernel writes every element, zeros where nothing survived the filter
+    dc = torch.full((V, D), float("nan"), dtype=gdt, device=dev)
     db = torch.zeros((V,), dtype=torch.float32, device=dev) if bias is not None else None
     counters = torch.zeros((4,), dtype=torch.int64, device=dev)
     ws = torch.empty((lib.cce_backward_workspace_bytes(B, V, D) // 8 + 1,), dtype=torch.int64, device=dev)
