@@ -12,10 +12,12 @@ from cut_cross_entropy.utils import TensorInfo
 
 
 # Upper bound of the dz chunk buffer of the unfiltered backward (bytes).  The chunk is [B, vc] in the input type
-# with vc a multiple of 256 classes, at most 16384; the library picks the vc that fits.  A smaller buffer means
-# more, smaller chunks: less memory, launches that fill the GPU less evenly and more passes over the dE
-# accumulator (measured, backward of E [15356, 4096] x C [128256, 4096]: 47.6 ms with 128 MB, 43.1 with 256,
-# 41.4 with 512; E [8192, 2048] x C [256000, 2048]: 24.0 / 22.6 / 22.6).
+# with vc a multiple of 256 classes, at most 16384; the library picks the vc that fits and fills the 256 compute
+# units most evenly.  A smaller buffer means more, smaller chunks: less memory, more launches and more passes over
+# the dE accumulator (measured, backward of E [15356, 4096] x C [128256, 4096]: 44.4 ms with 128 MB, 41.0 with
+# 256; E [8192, 2048] x C [256000, 2048]: 21.8 / 21.8; E [8192, 2304] x C [256000, 2304]: 24.8 / 25.7; with 32 MB
+# the last one takes 31.8).  On top of it comes, when dE is wanted in a 16-bit type, a [B, D] 16-bit
+# compensation buffer (dE is summed over the chunks as a pair of 16-bit numbers).
 DENSE_DZ_BYTES = 256 << 20
 
 # With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path pays for
@@ -33,6 +35,10 @@ DENSE_DZ_BYTES = 256 << 20
 # the soft-max is flat).  FILTERED_BACKWARD_PATH pins the choice: "sparse" or "dense" instead of "auto".
 DENSE_WHEN_FLAGGED_ABOVE = 0.17
 FILTERED_BACKWARD_PATH = "auto"
+# The unfiltered path's workspace (dz chunk + compensation buffer) grows with the number of rows; where memory
+# matters more than time, a byte count here keeps a FILTERED backward whose workspace would be larger on the
+# ownership kernels (which need one bit per 32 x 32 sub-tile and nothing else).  None: no limit.
+DENSE_WORKSPACE_LIMIT_BYTES: Optional[int] = None
 _OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
 
@@ -75,6 +81,9 @@ def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, fi
         return FILTERED_BACKWARD_PATH == "dense"
     if DENSE_WHEN_FLAGGED_ABOVE is None:
         return False
+    if (DENSE_WORKSPACE_LIMIT_BYTES is not None
+            and lib.cce_backward_dense_workspace_bytes(B, V, D, 1, DENSE_DZ_BYTES) > DENSE_WORKSPACE_LIMIT_BYTES):
+        return False
     key = (dev.index, V, D, dtype)
     with _monitors_lock:
         mon = _monitors.get(key)
@@ -88,8 +97,8 @@ def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, fi
 
 
 def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
-    """The unfiltered backward runs as (dz kernel + library GEMMs) when nothing that is asked for is
-    filtered and the layout suits the direct-to-LDS kernel."""
+    """The unfiltered backward (cce_backward_dense: dz chunks and the two products as MFMA kernels) runs when
+    nothing that is asked for is filtered and the layout suits the direct-to-LDS kernels."""
     if filter_eps_or_none(filter_eps) >= 0.0:
         if (want_de and filter_e_grad) or ((want_dc or want_dbias) and filter_c_grad):
             return False

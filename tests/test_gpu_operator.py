@@ -250,6 +250,16 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     assert len(calls) == 2
     monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "auto")
+    # a workspace limit below what the unfiltered path needs here keeps the ownership kernels; above, it does not
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 64 * 1024)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 2
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 64 << 20)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 3
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", None)
 
     g = torch.Generator().manual_seed(1)
     c2 = (torch.randn((65536, 128), generator=g) * 0.5).to(torch.bfloat16)  # 512 cells per row group, <= 32 hold a target
@@ -259,7 +269,7 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     for _ in range(2):
         linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
         torch.cuda.synchronize()
-    assert len(calls) == 2
+    assert len(calls) == 3
 
 
 @pytest.mark.parametrize("impl", ["cce", "cce_exact"])
