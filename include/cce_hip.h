@@ -218,10 +218,13 @@ int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int 
  * numbers, d_e itself and a compensation term in the workspace (the "Kahan" buffers of the reference's
  * cce_kahan* presets, :374-385: 16 bits of mantissa carried from chunk to chunk, d_e final after the last).
  *
- *   d_e      NULL or [n_rows, d], accumulated into (the caller zero-fills): float when d_e_is_fp32, else `dtype`;
- *            rows that are not valid tokens are not touched
+ *   d_e      NULL or [n_rows, d]: float when d_e_is_fp32 (accumulated into: the caller zero-fills), else `dtype`
+ *            (the rows of valid tokens are written, whatever they held); rows that are not valid tokens are
+ *            not touched in either case
  *   d_c      NULL or [v, d] with the strides of c; float when d_c_is_fp32 else `dtype`; written, not accumulated
- *   d_bias   NULL or [v] float, accumulated into
+ *   d_bias   NULL or [v] float, accumulated into.  The column sums run over dz as rounded to `dtype` (what the
+ *            products multiply); cce_backward and the reference (:253-256) sum dz before that rounding, so the
+ *            two differ by the rounding of each term (2^-9 relative for bf16, unbiased)
  *   workspace  256-byte aligned; at least cce_backward_dense_workspace_bytes(b, v, d, d_e in `dtype`, 0) bytes.
  *            Anything beyond that enlarges the chunks (fewer, better filled launches) up to 16384 classes.
  * Layout requirements as for cce_backward_dz (16-byte aligned e, c and d_e, unit stride_cd, row strides that
@@ -237,6 +240,25 @@ int cce_backward_dense(const void* e, const void* c, const void* bias,
                        float grad_scale, int d_e_is_fp32, int d_c_is_fp32,
                        int64_t shift, int64_t target_offset,
                        float softcap, int dtype, void* stream);
+
+/*
+ * The two matrix products of one vocabulary chunk on their own, for a caller that forms dz itself and wants
+ * fp32 results: the fp32 path of the Python host splits dz, c and e into 16-bit parts and sums the cross terms
+ * with one call per term.  The products of the reference's kernel (cut_cross_entropy/cce_backward.py:262-275
+ * and :289-302) as 16-bit-in, fp32-accumulate matrix products on the tiles cce_backward_dense runs, both in one
+ * launch:
+ *     d_e[i, :] += sum_v dz[i, v] c[v, :]                    i < b   (d_e: a [b, d] float accumulator, row stride ld_de)
+ *     d_c[v, :] (+)= sum_i dz[i, v] e[valids[i], :]          v < n_cls  (float, row stride ld_dc; added to when
+ *                                                            d_c_accumulate, else written)
+ *   dz   [b, ldz] in `dtype`; ldz >= n_cls rounded up to 64, and the columns up to there must hold finite values
+ *   c    [n_cls, d] row stride stride_cv (NULL when d_e is NULL);  e  [*, d] row stride stride_e (NULL when d_c is NULL)
+ * Pointers 16-byte aligned, ldz / stride_cv / stride_e multiples of 8, d a multiple of 8, ld_de / ld_dc multiples
+ * of 4; else CCE_ERR_MISALIGNED.
+ */
+int cce_backward_products(const void* dz, int64_t ldz, const void* c, int64_t stride_cv,
+                          const void* e, int64_t stride_e, const int32_t* valids,
+                          float* d_e, int64_t ld_de, float* d_c, int64_t ld_dc, int d_c_accumulate,
+                          int64_t b, int64_t n_cls, int64_t d, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -39,7 +39,10 @@ struct ProductParams {
   int64_t ld_de;        // row stride of d_e (elements)
   int first_chunk;      // nothing accumulated yet: the pair is written, not read
   void* d_c;            // first class of the chunk
+  int64_t ld_dc;        // row stride of d_c (elements)
   int dc_fp32;
+  int dc_accumulate;    // d_c (fp32) is added to, not written
+  int de_rows_by_number;  // the fp32 d_e is indexed by valid-row number (a [b, d] accumulator), not by row of e
   int64_t b;
   int d;
   int n_cls;            // classes in the chunk
@@ -98,7 +101,7 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
     const int64_t ri = m0 + row;          // valid-row number
     const int cg = n0 + col;
     if (ri >= p.b || cg >= p.d) return;
-    const int64_t re = (p.valids != nullptr) ? static_cast<int64_t>(p.valids[ri]) : ri;  // its row of e
+    const int64_t re = (p.valids != nullptr && !p.de_rows_by_number) ? static_cast<int64_t>(p.valids[ri]) : ri;  // its row of e
     if (!SPLIT_DE) {
       float4* dst = reinterpret_cast<float4*>(p.de_f32 + re * p.ld_de + cg);
       float4 a = dst[0], b = dst[1];
@@ -168,11 +171,17 @@ __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, in
     const int cls = m0 + row;
     const int cg = n0 + col;
     if (cls >= p.n_cls || cg >= p.d) return;
-    const int64_t off = static_cast<int64_t>(cls) * p.stride_cv + cg;
+    const int64_t off = static_cast<int64_t>(cls) * p.ld_dc + cg;
     if (p.dc_fp32) {
       float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.d_c) + off);
-      dst[0] = make_float4(v[0], v[1], v[2], v[3]);
-      dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+      float4 a = make_float4(v[0], v[1], v[2], v[3]), b = make_float4(v[4], v[5], v[6], v[7]);
+      if (p.dc_accumulate) {
+        const float4 a0 = dst[0], b0 = dst[1];
+        a.x += a0.x; a.y += a0.y; a.z += a0.z; a.w += a0.w;
+        b.x += b0.x; b.y += b0.y; b.z += b0.z; b.w += b0.w;
+      }
+      dst[0] = a;
+      dst[1] = b;
     } else {
       *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.d_c) + off) =
           make_uint4(Elem<T>::pack2(v[0], v[1]), Elem<T>::pack2(v[2], v[3]), Elem<T>::pack2(v[4], v[5]), Elem<T>::pack2(v[6], v[7]));
@@ -359,6 +368,9 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   p.de_lo = split_de ? static_cast<uint16_t*>(workspace) : nullptr;
   p.ld_de = stride_e;
   p.dc_fp32 = d_c_is_fp32;
+  p.ld_dc = stride_cv;
+  p.dc_accumulate = 0;
+  p.de_rows_by_number = 0;
   p.b = b;
   p.d = static_cast<int>(d);
 
@@ -421,5 +433,68 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   }
 #undef CCE_LAUNCH_PRODUCT
 
+  return status_from_hip(hipGetLastError());
+}
+
+// ---- the two products of one chunk on their own ----------------------------------------------------------------
+extern "C" int cce_backward_products(const void* dz, int64_t ldz, const void* c, int64_t stride_cv,
+                                     const void* e, int64_t stride_e, const int32_t* valids,
+                                     float* d_e, int64_t ld_de, float* d_c, int64_t ld_dc, int d_c_accumulate,
+                                     int64_t b, int64_t n_cls, int64_t d, int dtype, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (b < 0 || n_cls < 0 || d <= 0) return CCE_ERR_INVALID_ARGUMENT;
+  if (b == 0 || n_cls == 0) return CCE_OK;
+  if (dz == nullptr || (d_e != nullptr && c == nullptr) || (d_c != nullptr && e == nullptr)) return CCE_ERR_INVALID_ARGUMENT;
+  if (dtype != CCE_DTYPE_BF16 && dtype != CCE_DTYPE_F16) return CCE_ERR_UNSUPPORTED_DTYPE;
+  if (b >= (int64_t(1) << 31) - 512 || n_cls >= (int64_t(1) << 31) - 512 || d > (1 << 24)) return CCE_ERR_INVALID_ARGUMENT;
+  if (ldz >= (int64_t(1) << 30) || stride_cv >= (int64_t(1) << 30) || stride_e >= (int64_t(1) << 30))
+    return CCE_ERR_INVALID_ARGUMENT;
+  if (d_e == nullptr && d_c == nullptr) return CCE_OK;
+  if (!aligned16(dz) || ldz % 8 != 0 || ldz < (n_cls + 63) / 64 * 64 || d % 8 != 0) return CCE_ERR_MISALIGNED;
+  if (d_e != nullptr && (!aligned16(c) || stride_cv % 8 != 0 || !aligned16(d_e) || ld_de % 4 != 0 || ld_de < d))
+    return CCE_ERR_MISALIGNED;
+  if (d_c != nullptr && (!aligned16(e) || stride_e % 8 != 0 || !aligned16(d_c) || ld_dc % 4 != 0 || ld_dc < d))
+    return CCE_ERR_MISALIGNED;
+
+  ProductParams p;
+  p.dz = static_cast<const uint16_t*>(dz);
+  p.ldz = ldz;
+  p.c = static_cast<const uint16_t*>(c);
+  p.stride_cv = stride_cv;
+  p.e = static_cast<const uint16_t*>(e);
+  p.stride_e = stride_e;
+  p.valids = valids;
+  p.de_f32 = d_e;
+  p.de_hi = nullptr;
+  p.de_lo = nullptr;
+  p.ld_de = ld_de;
+  p.de_rows_by_number = 1;
+  p.first_chunk = 0;
+  p.d_c = d_c;
+  p.ld_dc = ld_dc;
+  p.dc_fp32 = 1;
+  p.dc_accumulate = d_c_accumulate;
+  p.b = b;
+  p.d = static_cast<int>(d);
+  p.n_cls = static_cast<int>(n_cls);
+  p.tiles_n = static_cast<int>((d + 255) / 256);
+  p.dc_tiles = (d_c != nullptr) ? static_cast<int>((n_cls + 255) / 256) * p.tiles_n : 0;
+  p.de_tiles = (d_e != nullptr) ? static_cast<int>((b + 255) / 256) * p.tiles_n : 0;
+  p.dc_per_xcd = (p.dc_tiles + 7) / 8;
+  p.de_per_xcd = (p.de_tiles + 7) / 8;
+  const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
+  const int lds = Tile4<BF16, true, true>::LDS_BYTES;
+  hipError_t err;
+  if (dtype == CCE_DTYPE_BF16) {
+    auto kern = dense_products_kernel<BF16, false>;
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (err != hipSuccess) return status_from_hip(err);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kProdThreads), lds, stream, p);
+  } else {
+    auto kern = dense_products_kernel<F16, false>;
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (err != hipSuccess) return status_from_hip(err);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kProdThreads), lds, stream, p);
+  }
   return status_from_hip(hipGetLastError());
 }

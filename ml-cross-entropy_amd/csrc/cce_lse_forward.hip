@@ -202,11 +202,6 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
     // One 32-row column block at a time, so that only 64 soft-capped logits are live at once.
     const int64_t vw0 = v0 + wv * (32 * kFwdWV);  // first class of this wave
     const float* wave_addend = addend + wv * (32 * kFwdWV);
-    float colsum[WANT_LA ? kFwdWV * 16 : 1];
-    if (WANT_LA) {
-#pragma unroll
-      for (int j = 0; j < kFwdWV * 16; ++j) colsum[j] = 0.0f;
-    }
 #pragma unroll
     for (int ti = 0; ti < kFwdWT; ++ti) {
       __builtin_amdgcn_sched_barrier(0);  // keep each column block's register use to itself
@@ -214,11 +209,25 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
       float bm[kFwdWV];  // this lane's maximum in each of the four 32-class blocks
       const float tm = column_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, half, s2, bm);
       if (WANT_LA) {
+        // Column sums over the 32 rows of this block, in natural-log units, added to the running average right
+        // away: nothing is carried from one column block to the next, so asking for the average costs the
+        // direct-to-LDS kernel no registers beyond these temporaries.
         const float ok = (t0 + wt * (32 * kFwdWT) + ti * 32 + l32 < p.b) ? 1.0f : 0.0f;
+        const float inv_b = kLn2 / static_cast<float>(p.b);
+        float* avg = p.logit_avg + vw0 + 4 * half;                 // this lane half's first class of the wave
+        const int left = static_cast<int>(min(p.v - vw0, static_cast<int64_t>(32 * kFwdWV))) - 4 * half;
 #pragma unroll
-        for (int vi = 0; vi < kFwdWV; ++vi)
+        for (int vi = 0; vi < kFwdWV; ++vi) {
+          __builtin_amdgcn_sched_barrier(0);  // one 32-class block at a time
 #pragma unroll
-          for (int r = 0; r < 16; ++r) colsum[vi * 16 + r] += (s2[vi][r] == -INFINITY) ? 0.0f : s2[vi][r] * ok;
+          for (int r = 0; r < 16; ++r) {
+            const int cls = vi * 32 + 8 * (r >> 2) + (r & 3);
+            float cs = (s2[vi][r] == -INFINITY) ? 0.0f : s2[vi][r] * ok;
+#pragma unroll
+            for (int off = 16; off >= 1; off >>= 1) cs += __shfl_xor(cs, off, 64);
+            if (l32 == 0 && cls < left) unsafeAtomicAdd(avg + cls, cs * inv_b);
+          }
+        }
       }
 
       if (p.tile_max != nullptr) {
@@ -247,21 +256,6 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
       m2[ti] = mn;
     }
 
-    if (WANT_LA) {
-      // column sums over the rows of this wave, in natural-log units
-      const float inv_b = kLn2 / static_cast<float>(p.b);
-#pragma unroll
-      for (int vi = 0; vi < kFwdWV; ++vi) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t vg = vw0 + vi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          float cs = colsum[vi * 16 + r];
-#pragma unroll
-          for (int off = 16; off >= 1; off >>= 1) cs += __shfl_xor(cs, off, 64);
-          if (l32 == 0 && vg < p.v) unsafeAtomicAdd(p.logit_avg + vg, cs * inv_b);
-        }
-      }
-    }
   }
 
   // ---- merge the two lane halves, then the two wave rows, and emit one partial per row -------
@@ -320,7 +314,7 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
   const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
-  const bool fast = aligned && (p.d % kDmaBK == 0) && !want_la;
+  const bool fast = aligned && (p.d % kDmaBK == 0);
   const bool general = want_la || (p.bias != nullptr) || (p.v % Tile::TILE_V != 0);
   const int grid = p.items_per_xcd * 8;
   hipError_t err;
@@ -333,7 +327,9 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                           \
   } while (0)
   if (fast) {
-    if (general) CCE_LAUNCH_FWD(true, true, true, false); else CCE_LAUNCH_FWD(true, true, false, false);
+    if (want_la) CCE_LAUNCH_FWD(true, true, true, true);
+    else if (general) CCE_LAUNCH_FWD(true, true, true, false);
+    else CCE_LAUNCH_FWD(true, true, false, false);
   } else if (aligned) {
     if (want_la) CCE_LAUNCH_FWD(false, true, true, true); else CCE_LAUNCH_FWD(false, true, true, false);
   } else {

@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
 STAT_ROWS = 32
 STAT_COLS = 32
@@ -57,6 +57,10 @@ _SIGNATURES = {
         _i32,
         [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64]
         + [_i64] * 4 + [_i64] * 3 + [_f32, _i32, _i32, _i64, _i64, _f32, _i32, _ptr],
+    ),
+    "cce_backward_products": (
+        _i32,
+        [_ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _i64, _ptr, _i64, _i32, _i64, _i64, _i64, _i32, _ptr],
     ),
     "cce_backward_dz": (
         _i32,

@@ -223,7 +223,12 @@ def cce_backward_kernel(
         # (dC, dBias) or summed over the chunks in an fp32 workspace (dE): no fp32 gradient buffers are needed
         de_dtype, dc_dtype = e_info.dtype, c_info.dtype
     n_valid_rows = valids.size(0) if valids is not None else e.size(0)
-    de = torch.zeros_like(e, dtype=de_dtype) if e_info.requires_grad else None
+    de = None
+    if e_info.requires_grad:
+        # the unfiltered path writes every valid row of a 16-bit dE; rows outside `valids` and every other case
+        # (the ownership kernels, an fp32 accumulator) start from zeros
+        de_written_whole = dense and valids is None and de_dtype != torch.float32 and n_valid_rows > 0
+        de = torch.empty_like(e, dtype=de_dtype) if de_written_whole else torch.zeros_like(e, dtype=de_dtype)
     dc = None
     if c_info.requires_grad:
         # both paths write every element of dC (the ownership kernel stores zeros for a class group nothing

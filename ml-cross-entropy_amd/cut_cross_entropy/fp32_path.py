@@ -14,14 +14,16 @@ three parts of the bias in C').  The vocabulary is walked in chunks so that the 
 classifier stays small; chunk log-sum-exps are merged with logaddexp.
 
 Backward: the gradient filter threshold of fp32 is far below anything a soft-max produces, so the
-backward is the unfiltered one: the dz kernel runs on the widened matrices and writes dz as fp32, and
-the two products are fp32 GEMMs on the original matrices (split-part GEMMs were measured slower than the
-library's fp32 GEMM once the splitting passes are counted: 75 against 117 TFLOP/s).
+backward is the unfiltered one: the dz kernel runs on the widened matrices and writes the dz of a vocabulary
+chunk as fp32; dz, the classifier chunk and the rows of e are split into the same three parts, and the two
+products dE += dz . C and dC = dz^T . E are summed over the same cross terms, one call of the library's 16-bit
+product kernels per term (``cce_backward_products``: fp32 accumulators, dE and dC added to in fp32).  No copy
+of an operand is widened for this: a term pairs part i of dz with part j of C and of E as they lie.
 
 ``torch.set_float32_matmul_precision``: "highest" (the default) takes the six terms above; with "high" or
 "medium" the caller has asked for fast fp32 products (the reference then lets Triton use tf32, 10 mantissa
-bits, cce_lse_forward.py:129-131) and the logits are formed from the three leading terms hi*hi + hi*mid +
-mid*hi (16 bits), half the work; the fp32 GEMMs of the backward follow the same switch inside the library.
+bits, cce_lse_forward.py:129-131) and logits and gradient products are formed from the three leading terms
+hi*hi + hi*mid + mid*hi (16 bits), half the work.
 """
 
 from typing import Optional, Tuple
@@ -119,10 +121,14 @@ def fp32_indexed_neg_dot(e, c, bias, targets, valids, shift, softcap, target_off
     return torch.where(ok, -logit, torch.zeros_like(logit))
 
 
+def _pad_cols(x: torch.Tensor, width: int) -> torch.Tensor:
+    return x if x.size(1) == width else torch.nn.functional.pad(x, (0, width - x.size(1)))
+
+
 def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offset, softcap, grad_scale,
                   want_de, want_dc, want_dbias):
-    """(dE, dC, dBias) in fp32: dz of a vocabulary chunk from the HIP kernel (fp32 output), products as
-    fp32 GEMMs."""
+    """(dE, dC, dBias) in fp32: dz of a vocabulary chunk from the HIP kernel (fp32 output), then the two
+    products as sums of 16-bit cross terms on the library's product kernels."""
     lib = _hip.load()
     dev = e.device
     n, d = e.shape
@@ -135,18 +141,29 @@ def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offs
     if n_valid == 0 or not (want_de or want_dc or want_dbias):
         return de, dc, dbias
     terms = n_terms()
+    bf16 = _hip.DTYPE_CODES[torch.bfloat16]
     e6 = widen_e(e, bias is not None, terms)
-    e_rows = e if rows is None else e.index_select(0, rows)
-    de_acc = torch.zeros((n_valid, d), dtype=torch.float32, device=dev) if want_de else None
+    d8 = (d + 7) // 8 * 8  # the product kernels move 16-byte pieces
+    e_parts = None
+    if want_dc:
+        e_rows = e if rows is None else e.index_select(0, rows)
+        e_parts = [_pad_cols(part, d8).contiguous() for part in split3(e_rows)]
+    de_acc = torch.zeros((n_valid, d8), dtype=torch.float32, device=dev) if want_de else None
     vc = min(_chunk(v, e6.size(1) * 2, _WIDE_C_BYTES), _chunk(v, n_valid * 4, _DZ_ELEMS * 4))
-    dz_buf = torch.empty((n_valid * ((min(vc, v) + 3) // 4 * 4),), dtype=torch.float32, device=dev)
+    ldz_full = (min(vc, v) + 63) // 64 * 64
+    # fp32 dz of a chunk; its padding columns are never written by the kernel and have to read as zeros
+    dz_buf = torch.zeros((n_valid * ldz_full,), dtype=torch.float32, device=dev)
+    dc_direct = dc is not None and d8 == d and dc.is_contiguous()
+    dc_tmp = None if (dc is None or dc_direct) else torch.empty((min(vc, v), d8), dtype=torch.float32, device=dev)
     do = do.to(torch.float32).contiguous().view(-1)
     dlse = dlse.to(torch.float32).contiguous().view(-1) if dlse is not None else None
     targets = targets.to(torch.int64).contiguous()
     stream = _hip.current_stream_ptr(dev)
     for v0 in range(0, v, vc):
         m = min(vc, v - v0)
-        ldz = (m + 3) // 4 * 4
+        ldz = (m + 63) // 64 * 64
+        if ldz != ldz_full:
+            dz_buf.zero_()  # the last, shorter chunk lays the buffer out anew
         dz = dz_buf[: n_valid * ldz].view(n_valid, ldz)
         c_chunk = c[v0 : v0 + m]
         c6 = widen_c(c_chunk, bias[v0 : v0 + m] if bias is not None else None, terms)
@@ -159,19 +176,35 @@ def fp32_backward(e, c, bias, lse, do, dlse, valids, targets, shift, target_offs
                 n, n_valid, m, e6.size(1),
                 e6.stride(0), c6.stride(0), c6.stride(1),
                 float(grad_scale), int(shift), int(target_offset) + v0,
-                float(softcap) if softcap is not None else 0.0, _hip.DTYPE_CODES[torch.bfloat16], stream,
+                float(softcap) if softcap is not None else 0.0, bf16, stream,
             )
         _hip.check(status, "cce_backward_dz")
-        dzv = dz[:, :m]
-        if de_acc is not None:
-            de_acc.addmm_(dzv, c_chunk)
-        if dc is not None:
-            torch.mm(dzv.t(), e_rows, out=dc[v0 : v0 + m])
+        del c6
         if dbias is not None:
-            dbias[v0 : v0 + m] = dzv.sum(dim=0)
+            dbias[v0 : v0 + m] = dz[:, :m].sum(dim=0)
+        if de_acc is None and dc is None:
+            continue
+        dz_parts = split3(dz)
+        c_parts = [_pad_cols(part, d8).contiguous() for part in split3(c_chunk)] if de_acc is not None else None
+        dc_out = None
+        if dc is not None:
+            dc_out = dc[v0 : v0 + m] if dc_direct else dc_tmp[:m]
+        for k in range(terms):
+            a, b = dz_parts[_E_PARTS[k]], _C_PARTS[k]
+            with torch.cuda.device(dev):
+                status = lib.cce_backward_products(
+                    a.data_ptr(), ldz,
+                    c_parts[b].data_ptr() if c_parts is not None else None, d8,
+                    e_parts[b].data_ptr() if e_parts is not None else None, d8, None,
+                    _hip.ptr(de_acc), d8, _hip.ptr(dc_out), d8, 1 if k > 0 else 0,
+                    n_valid, m, d8, bf16, stream,
+                )
+            _hip.check(status, "cce_backward_products")
+        if dc is not None and not dc_direct:
+            dc[v0 : v0 + m] = dc_tmp[:m, :d]
     if de is not None:
         if rows is None:
-            de.copy_(de_acc)
+            de.copy_(de_acc[:, :d])
         else:
-            de.index_copy_(0, rows, de_acc)
+            de.index_copy_(0, rows, de_acc[:, :d].contiguous())
     return de, dc, dbias

@@ -374,3 +374,48 @@ def test_entry_points_reject_bad_arguments_before_launching():
     torch.cuda.synchronize()
     assert (de == 0).all() and (dc == 0).all()
     assert lib.cce_error_string(INVALID) and lib.cce_error_string(MISALIGNED) and lib.cce_error_string(DTYPE)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (300, 500, 72), (1000, 130, 264), (33, 64, 8)])
+def test_backward_products_abi(dtype, shape):
+    """cce_backward_products: d_e += dz . c and d_c (+)= dz^T . e[valids] with fp32 results, against the same
+    products in fp64 of the same 16-bit inputs (exact up to fp32 accumulation: 1e-5 of the row scale)."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    B, M, D = shape
+    g = torch.Generator().manual_seed(B + M + D)
+    n_rows = B + 37
+    ldz = (M + 63) // 64 * 64
+    dz = torch.zeros((B, ldz), dtype=dtype)
+    dz[:, :M] = (torch.randn((B, M), generator=g) * 0.1).to(dtype)
+    c = torch.randn((M, D), generator=g).to(dtype)
+    e = torch.randn((n_rows, D), generator=g).to(dtype)
+    valids = torch.randperm(n_rows, generator=g)[:B].sort().values.to(torch.int32)
+    de0 = torch.randn((B, D), generator=g)
+    dc0 = torch.randn((M, D), generator=g)
+    want_de = de0.double() + dz[:, :M].double() @ c.double()
+    prod_dc = dz[:, :M].double().T @ e[valids.long()].double()
+    code = 0 if dtype == torch.bfloat16 else 1
+    dzd, cd, ed, vd = dz.to(dev), c.to(dev), e.to(dev), valids.to(dev)
+    for accumulate in (0, 1):
+        ded, dcd = de0.to(dev), dc0.to(dev)
+        st = lib.cce_backward_products(dzd.data_ptr(), ldz, cd.data_ptr(), D, ed.data_ptr(), D, vd.data_ptr(),
+                                       ded.data_ptr(), D, dcd.data_ptr(), D, accumulate, B, M, D, code,
+                                       torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.cce_error_string(st)
+        torch.cuda.synchronize()
+        want_dc = prod_dc + (dc0.double() if accumulate else 0.0)
+        for got, want in ((ded, want_de), (dcd, want_dc)):
+            scale = want.abs().max().item()
+            assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * scale
+    # one product alone, and the layout checks
+    ded = de0.to(dev)
+    st = lib.cce_backward_products(dzd.data_ptr(), ldz, cd.data_ptr(), D, None, 0, None, ded.data_ptr(), D, None, 0, 0,
+                                   B, M, D, code, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert (ded.cpu().double() - want_de).abs().max().item() <= 1e-5 * want_de.abs().max().item()
+    st = lib.cce_backward_products(dzd.data_ptr(), M if M % 64 else ldz - 8, cd.data_ptr(), D, None, 0, None,
+                                   ded.data_ptr(), D, None, 0, 0, B, M, D, code, torch.cuda.current_stream().cuda_stream)
+    assert st != 0  # dz rows shorter than the reduction rounded up to 64

@@ -194,6 +194,10 @@ def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids
         ed = e.cuda().requires_grad_(True)
         cd = c.cuda().requires_grad_(True)
         loss = linear_cross_entropy(ed, cd, t.cuda(), softcap=25.0, impl=impl, shift=1 if with_valids else 0)
+        # the gradients are allocated without a fill where the kernels write them whole: give the allocator
+        # blocks full of NaN to hand out
+        for numel in (e.numel(), c.numel(), 384 * 128, 1100 * 128):
+            torch.full((numel,), float("nan"), dtype=torch.bfloat16, device="cuda")
         loss.backward()
         e64 = e.double().requires_grad_(True)
         c64 = c.double().requires_grad_(True)
