@@ -178,9 +178,10 @@ int cce_count_flagged_cells(const float* tile_max, const float* lse, int64_t b, 
  * logit recompute :170-188, softmax minus one-hot :196-207, d_out / d_lse scaling :238-248,
  * soft-cap gradient :251, rounding to the input type :256) with the gradient filter off.  What the
  * reference does next inside the same kernel -- the two products d_e += dz . c (:262-275) and
- * d_c += dz^T . e (:289-302), through atomics -- is left to the caller: with every dz in play they
- * are plain GEMMs (d_e[rows] += dz . c, d_c = dz^T . e[rows], d_bias = column sums of dz) on the
- * [b, v] matrix this function fills, chunk of the vocabulary by chunk.
+ * d_c += dz^T . e (:289-302), through atomics -- is not done here: with every dz in play they are dense
+ * matrix products (d_e[rows] += dz . c, d_c = dz^T . e[rows], d_bias = column sums of dz) on the [b, v] matrix
+ * this function fills, chunk of the vocabulary by chunk.  cce_backward_dense runs dz and products in one call,
+ * cce_backward_products the products alone.
  *
  *   c, bias    the chunk's rows: v classes starting at the caller's offset
  *   lse        [b] float, the LSE over the WHOLE vocabulary

@@ -47,8 +47,9 @@ struct ProductParams {
   int d;
   int n_cls;            // classes in the chunk
   int tiles_n;          // column tiles of either output
-  int dc_tiles, dc_per_xcd;  // tiles of dC (first in the grid: the longer reductions start first), per XCD slot count
+  int dc_tiles, dc_per_xcd;  // tiles of dC, slots per XCD
   int de_tiles, de_per_xcd;
+  int de_first;              // the dE tiles have the longer reduction and take the first block ids
 };
 
 constexpr int kProdThreads = 256;  // four waves, one per SIMD
@@ -189,19 +190,21 @@ __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, in
   });
 }
 
-// Both products of one chunk in one launch: the dC tiles (reduction over all B rows) take the first block ids,
-// the dE tiles (reduction over the classes of the chunk) the rest.  Blocks are handed to compute units in id
-// order as units fall free, so the two kinds fill each other's last round.
+// Both products of one chunk in one launch.  Blocks are handed to compute units in id order as units fall free:
+// the kind of tile with the longer reduction (dC: all B rows; dE: the classes of the chunk) takes the first block
+// ids, so that the shorter tiles fill the last round of the longer ones.
 template <typename T, bool SPLIT_DE>
 __global__ __launch_bounds__(kProdThreads, 1) void dense_products_kernel(ProductParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int dc_blocks = p.dc_per_xcd * 8;
+  const int first_blocks = (p.de_first ? p.de_per_xcd : p.dc_per_xcd) * 8;
+  const bool first = static_cast<int>(blockIdx.x) < first_blocks;
+  const int block = first ? blockIdx.x : blockIdx.x - first_blocks;
   int tm, tn;
-  if (static_cast<int>(blockIdx.x) < dc_blocks) {
-    if (!product_tile_of(blockIdx.x, p.dc_tiles, p.dc_per_xcd, p.tiles_n, tm, tn)) return;
+  if (first != (p.de_first != 0)) {
+    if (!product_tile_of(block, p.dc_tiles, p.dc_per_xcd, p.tiles_n, tm, tn)) return;
     dense_dc_tile<T>(p, tm, tn, smem);
   } else {
-    if (!product_tile_of(blockIdx.x - dc_blocks, p.de_tiles, p.de_per_xcd, p.tiles_n, tm, tn)) return;
+    if (!product_tile_of(block, p.de_tiles, p.de_per_xcd, p.tiles_n, tm, tn)) return;
     dense_de_tile<T, SPLIT_DE>(p, tm, tn, smem);
   }
 }
@@ -255,10 +258,11 @@ static double product_makespan(int64_t n_long, int64_t len_long, int64_t n_short
   return static_cast<double>(worst);
 }
 
-// Classes per chunk for a dz buffer of at most `max_dz_bytes`: a multiple of 256 up to 8192 that the buffer can
-// hold, chosen for the least estimated time per class: the dz kernel and the product launch (dC tiles with a
-// reduction over b rows, dE tiles with a reduction over vc classes, filling 256 compute units in rounds) plus a
-// fixed cost per launch that favours few, large chunks.  0: the buffer cannot hold 256 classes.
+// Classes per chunk for a dz buffer of at most `max_dz_bytes`: a multiple of 256 up to 16384 that the buffer can
+// hold, chosen for the least estimated time of the whole vocabulary (whole chunks and the shorter last one): per
+// chunk the dz kernel and the product launch (dC tiles with a reduction over b rows, dE tiles with a reduction
+// over vc classes, the longer kind first, filling 256 compute units as they fall free).  0: the buffer cannot
+// hold 256 classes.
 static int64_t dense_chunk_classes(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de, bool want_dc) {
   // the same question comes with every step of a training loop: remember the last answer of this thread
   struct Memo {
@@ -273,6 +277,18 @@ static int64_t dense_chunk_classes(int64_t b, int64_t v, int64_t d, int64_t max_
   return answer;
 }
 
+// Estimated time of one chunk of vc classes in units of 256 reduction steps of a tile: the dz kernel (row_tiles x
+// vc / 256 logit tiles of d / 256 units each, in rounds of 256) and the product launch.
+static double chunk_cost(int64_t b, int64_t d, int64_t vc, bool want_de, bool want_dc) {
+  const int64_t col_tiles = (d + 255) / 256;
+  const int64_t row_tiles = (b + 255) / 256;
+  const double products = product_makespan(want_dc ? vc / 256 * col_tiles : 0, row_tiles,
+                                           want_de ? row_tiles * col_tiles : 0, vc / 256);
+  const int64_t dz_tiles = row_tiles * (vc / 256);
+  const double dz = static_cast<double>((dz_tiles + 255) / 256) * static_cast<double>(col_tiles);
+  return products + dz + 0.25;  // the constant only breaks ties towards fewer chunks: launches queue back to back
+}
+
 static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int64_t max_dz_bytes, bool want_de,
                                             bool want_dc) {
   const int64_t v_pad = (v + 255) / 256 * 256;
@@ -280,23 +296,14 @@ static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int
   if (top > 16384) top = 16384;
   if (top < 256) return 0;
   if (top >= v_pad) return v_pad;
-  const int64_t col_tiles = (d + 255) / 256;
-  const int64_t row_tiles = (b + 255) / 256;
   int64_t best = top;
   double best_cost = 1e300;
   for (int64_t vc = top; vc >= 256; vc -= 256) {
-    const int64_t chunks = (v + vc - 1) / vc;
-    const double products = product_makespan(want_dc ? vc / 256 * col_tiles : 0, (b + 255) / 256,
-                                             want_de ? row_tiles * col_tiles : 0, vc / 256);
-    // dz: row_tiles x (vc / 256) logit tiles of d / 256 units each, in rounds of 256 as well
-    const int64_t dz_tiles = row_tiles * (vc / 256);
-    const double dz = static_cast<double>((dz_tiles + 255) / 256) * static_cast<double>(col_tiles);
-    // One unit (256 reduction steps of a tile) is about 3.9 us.  Per chunk: two launches with their gaps, fill and
-    // drain (~ 10 us each), and the read-modify-write of the fp32 dE accumulator (b x d x 8 bytes at ~ 3.5 TB/s),
-    // which all tiles of a round do at the same time.
-    const double per_launch = 2.5;
-    const double rmw = want_de ? static_cast<double>(b) * static_cast<double>(d) * 8.0 / 3.5e12 / 3.9e-6 : 0.0;
-    const double cost = static_cast<double>(chunks) * (products + dz + 2.0 * per_launch + rmw);
+    // whole chunks, then the shorter last one
+    const int64_t full = v / vc;
+    const int64_t rest = (v - full * vc + 255) / 256 * 256;
+    double cost = static_cast<double>(full) * chunk_cost(b, d, vc, want_de, want_dc);
+    if (rest > 0) cost += chunk_cost(b, d, rest, want_de, want_dc);
     if (cost < best_cost * (1.0 - 1e-9)) {
       best = vc;
       best_cost = cost;
@@ -409,6 +416,7 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
     p.dc_per_xcd = (p.dc_tiles + 7) / 8;
     p.de_tiles = (d_e != nullptr) ? static_cast<int>((b + 255) / 256) * tiles_n : 0;
     p.de_per_xcd = (p.de_tiles + 7) / 8;
+    p.de_first = (n > b) ? 1 : 0;
     const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
     if (blocks > 0) {
       if (dtype == CCE_DTYPE_BF16) {
@@ -482,6 +490,7 @@ extern "C" int cce_backward_products(const void* dz, int64_t ldz, const void* c,
   p.de_tiles = (d_e != nullptr) ? static_cast<int>((b + 255) / 256) * p.tiles_n : 0;
   p.dc_per_xcd = (p.dc_tiles + 7) / 8;
   p.de_per_xcd = (p.de_tiles + 7) / 8;
+  p.de_first = (n_cls > b) ? 1 : 0;
   const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
   const int lds = Tile4<BF16, true, true>::LDS_BYTES;
   hipError_t err;

@@ -1,8 +1,8 @@
 // cce_backward_dz: the gradient of the loss with respect to the logits of one vocabulary chunk,
 //     dz[i, j] = (p_ij (g_i + h_i) - [j == target_i] g_i) (1 - tanh^2)      p_ij = exp(s_ij - lse_i)
-// written to HBM in the input type, for the unfiltered ("exact") backward: with every entry of the
-// gradient in play the two products dE = dz . C and dC = dz^T . E are plain GEMMs, and the caller runs
-// them as such on the chunk.  The kernel is the forward kernel with another epilogue: same work
+// written to memory in the input type (or as fp32), for the unfiltered ("exact") backward: with every entry of
+// the gradient in play the two products dE = dz . C and dC = dz^T . E are dense matrix products over the chunk,
+// which the kernels of cce_backward_dense.hip run.  The kernel is the forward kernel with another epilogue: same work
 // items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as whole rows
 // of 256 bytes per wave instruction after a transposition through LDS.
 #include "cce_dense.h"
