@@ -120,7 +120,8 @@ int cce_indexed_neg_dot(const void* e, const void* c, const int64_t* targets, co
                         float softcap, int dtype, void* stream);
 
 /* Scratch bytes cce_backward needs: one survivor bit per 32 x 32 sub-tile, each 32-row group's bits
- * padded to whole 32-bit words. */
+ * padded to whole 32-bit words, then a count and one int32 per 32-class group (the class groups its second,
+ * full dC pass takes over from the light one). */
 int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d);
 
 /*

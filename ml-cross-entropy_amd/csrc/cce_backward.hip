@@ -50,6 +50,8 @@ struct BwdParams {
   float grad_scale, filter_eps, log_eps;
   int filter_e, filter_c, d_out_is_scalar, de_fp32, dc_fp32;
   int shortcut;  // tile_max may be used to skip cells before the recompute
+  int light_on;  // dC pass: class groups with at most kFLightMaxEntries entries are left to the light variant
+  int* heavy_list;  // [1 + nvg]: count, then the class groups the light variant leaves to the full one
   int ntg, nvc, nvg, bit_words, nslices, dslice, stat_cols;
   int vec_e, vec_c;  // 4-element vector stores are legal for dE / dC
   Softcap sc;
@@ -619,15 +621,24 @@ constexpr int kFOtherBytes = 128 * kFRowBytes;      // 32 KB
 constexpr int kFOwnBytes = 32 * kFRowBytes;         //  8 KB
 constexpr int kFStageBytes = kFOtherBytes + kFOwnBytes;
 constexpr int kFMaxChunks = 18;                     // 18 * 128 = 2304 columns of D per workgroup
-constexpr int kFOffDz = 3 * kFStageBytes;           // 120 KB
-constexpr int kFOffList = kFOffDz + 8 * 1024;       //   8 KB entry list (2048 entries)
-constexpr int kFOffFlag = kFOffList + 8 * 1024 + 16; // 512 B (the list holds 2048 entries + 3 carried over)
-constexpr int kFOffBits = kFOffFlag + 512;          //   8 KB
-constexpr int kFOffMeta = kFOffBits + kMaxBitWords * 4;
-constexpr int kFLdsBytes = kFOffMeta + 5 * kMetaRows * 4 + 32 * 4 + 128 * 4 + 128 * 4 + 64;
+// LDS layout.  LIGHT (the dC pass of class groups with at most two entries, below): a 48 KB ring and no
+// survivor-bit row, 68 KB in all, so that two workgroups share a compute unit.
+template <bool LIGHT>
+struct FastLds {
+  static constexpr int kRing = LIGHT ? 48 * 1024 : 3 * kFStageBytes;  // 48 KB / 120 KB
+  static constexpr int kOffDz = kRing;                   //   8 KB dz [own][other]
+  static constexpr int kOffList = kOffDz + 8 * 1024;     //   8 KB entry list (2048 entries + 3 carried over)
+  static constexpr int kOffFlag = kOffList + 8 * 1024 + 16;  // 512 B per-cell sub-block masks (dE)
+  static constexpr int kOffBits = kOffFlag + 512;        //   8 KB survivor-bit row (dE)
+  static constexpr int kOffMeta = kOffBits + (LIGHT ? 0 : kMaxBitWords * 4);
+  static constexpr int kBytes = kOffMeta + 5 * kMetaRows * 4 + 32 * 4 + 128 * 4 + 128 * 4 + 64;
+};
+constexpr int kFLdsBytes = FastLds<false>::kBytes;
+constexpr int kFLightLdsBytes = FastLds<true>::kBytes;
+constexpr int kFLightMaxEntries = 2;                // entries of a class group the light dC pass takes on
 constexpr int kFSegCells = 512;                     // dE: cells scanned per pass (<= 2048 entries)
 constexpr int kFListCap = 2048;
-static_assert(kFLdsBytes <= 160 * 1024, "LDS budget of gfx950");
+static_assert(kFLdsBytes <= 160 * 1024 && 2 * kFLightLdsBytes <= 160 * 1024, "LDS budget of gfx950");
 
 template <typename T>
 __device__ __forceinline__ typename Elem<T>::vec8 fstage_frag(const unsigned char* lds, int row, int chunk) {
@@ -673,15 +684,17 @@ __device__ __forceinline__ void wait_vmcnt_upto(int n) {
   }
 }
 
-template <typename T, bool IS_DE>
-__global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParams p) {
+template <typename T, bool IS_DE, bool LIGHT = false>
+__global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_kernel(BwdParams p) {
+  static_assert(!(LIGHT && IS_DE), "the light variant is a dC pass");
+  using Lds = FastLds<LIGHT>;
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sDz = smem + kFOffDz;
-  int* sList = reinterpret_cast<int*>(smem + kFOffList);
-  unsigned char* sFlag = smem + kFOffFlag;
-  uint32_t* sBits = reinterpret_cast<uint32_t*>(smem + kFOffBits);
+  unsigned char* sDz = smem + Lds::kOffDz;
+  int* sList = reinterpret_cast<int*>(smem + Lds::kOffList);
+  unsigned char* sFlag = smem + Lds::kOffFlag;
+  uint32_t* sBits = reinterpret_cast<uint32_t*>(smem + Lds::kOffBits);
   RowMeta meta;
-  meta.row = reinterpret_cast<int*>(smem + kFOffMeta);
+  meta.row = reinterpret_cast<int*>(smem + Lds::kOffMeta);
   meta.tgt = meta.row + kMetaRows;
   meta.lse2 = reinterpret_cast<float*>(meta.tgt + kMetaRows);
   meta.g = meta.lse2 + kMetaRows;
@@ -697,8 +710,14 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int half = lane >> 5;
-  const int own = blockIdx.x / p.nslices;
+  int own = blockIdx.x / p.nslices;
   const int slice = blockIdx.x % p.nslices;
+  if (IS_DE && blockIdx.x == 0 && threadIdx.x == 0 && p.heavy_list != nullptr) p.heavy_list[0] = 0;  // for the dC passes
+  if (!IS_DE && !LIGHT && p.light_on) {
+    // the full dC pass after the light one: only the class groups that one listed
+    if (own >= p.heavy_list[0]) return;
+    own = p.heavy_list[1 + own];
+  }
   const int d_begin = slice * p.dslice;
   const int d_end = min(static_cast<int>(p.d), d_begin + p.dslice);
   const int nchunks = (d_end - d_begin) / kFCols;
@@ -746,11 +765,28 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
   }
 
   // wave w owns columns [32 w, 32 w + 32) of every 128-column chunk
-  f32x16 acc[kFMaxChunks];
+  // (the light variant keeps no gradient between chunks: one trip at most, every chunk leaves as it is formed)
+  constexpr int kAccChunks = LIGHT ? 1 : kFMaxChunks;
+  f32x16 acc[kAccChunks];
 #pragma unroll
-  for (int ci = 0; ci < kFMaxChunks; ++ci)
+  for (int ci = 0; ci < kAccChunks; ++ci)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[ci][r] = 0.0f;
+
+  // light variant: the 32 own rows x 128 columns of one chunk, 16-bit, straight from the accumulator block of
+  // this wave (lane = own row, registers = 4 x 4 consecutive columns)
+  auto store_chunk_direct = [&](int ci, const f32x16& a) {
+    const int id = own_ids[l32];
+    if (id < 0) return;
+    uint16_t* dst = static_cast<uint16_t*>(p.d_c) + static_cast<int64_t>(id) * own_sr + d_begin + ci * kFCols + wave * 32 + 4 * half;
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      uint2 pk;
+      pk.x = Elem<T>::pack2(a[r4 * 4 + 0], a[r4 * 4 + 1]);
+      pk.y = Elem<T>::pack2(a[r4 * 4 + 2], a[r4 * 4 + 3]);
+      *reinterpret_cast<uint2*>(dst + 8 * r4) = pk;
+    }
+  };
 
   unsigned long long n_recomputed = 0, n_product = 0;
   bool touched = false;
@@ -824,6 +860,11 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       __syncthreads();
     }
     const int list_n = use_list ? sMisc[0] : (IS_DE ? seg_n * 4 : seg_n);
+    // Class groups with few entries belong to the light variant when it runs (p.light_on, one segment only).
+    if (LIGHT && list_n > kFLightMaxEntries) {
+      if (tid == 0) p.heavy_list[1 + atomicAdd(p.heavy_list, 1)] = own;
+      return;
+    }
     // A class group nothing survived for goes straight to writing its zeros.
     if (!IS_DE && list_n == 0 && n_units <= seg_units) break;
     // Only the last segment runs a trip that is not full: what is left over goes to the front of the next list.
@@ -880,7 +921,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
       // stage holds the rows of the present entries followed by the own rows.
       const int own_off = 32 * nent * kFRowBytes;
       const int slot_bytes = own_off + kFOwnBytes;
-      const int ring = (nent >= 3) ? 3 : ((nent == 2) ? 5 : 7);  // slots of this size in the 120 KB ring
+      const int ring = Lds::kRing / slot_bytes;  // slots of this size in the ring: 3 / 5 / 7 (light: 2 / 3)
       const int ahead = ring - 1;                              // stages in flight
       // load q of this wave for the stage that starts at column col0: q < 8 other side, q = 8, 9 own side
       auto issue_load = [&](int q, int col0, int slot, bool with_own, uint32_t entries) {
@@ -910,7 +951,7 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
         constexpr int NKK = 8 / KPARTS;
         constexpr int OWN_OFF = 32 * NENT * kFRowBytes;
         constexpr int SLOT = OWN_OFF + kFOwnBytes;
-        constexpr int RING = (NENT >= 3) ? 3 : ((NENT == 2) ? 5 : 7);
+        constexpr int RING = Lds::kRing / SLOT;
         constexpr int AHEAD = RING - 1;
         constexpr int PER_STAGE = 2 * NENT + 2;
         auto issue = [&](auto q_tag, int col0, unsigned base) {
@@ -986,9 +1027,13 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
           slot = (slot + 1 == RING) ? 0 : slot + 1;
         }
       };
-      if (nent >= 3) logits_of_trip(std::integral_constant<int, 4>{});
-      else if (nent == 2) logits_of_trip(std::integral_constant<int, 2>{});
-      else logits_of_trip(std::integral_constant<int, 1>{});
+      if (nent >= 3) {
+        if constexpr (!LIGHT) logits_of_trip(std::integral_constant<int, 4>{});
+      } else if (nent == 2) {
+        logits_of_trip(std::integral_constant<int, 2>{});
+      } else {
+        logits_of_trip(std::integral_constant<int, 1>{});
+      }
       mfma_drain(s);
       __syncthreads();  // every load has landed and every stage is consumed
       if (kparts > 1) {  // partial logits -> the owner, through the idle ring, in a fixed order
@@ -1070,32 +1115,48 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 #pragma unroll 1
         for (int j = 0; j < npre; ++j) issue_stage(d_begin + j * kFCols, j, false, mask);
         int pslot = 0;  // ci % ring
+        auto product_chunk = [&](int ci, f32x16& accum, auto in_agpr) {
+          wait_vmcnt_upto(min(ahead - 1, nchunks - 1 - ci) * 2 * nused);  // the stages after ci may be in flight
+          __syncthreads();
+          const unsigned char* so = smem + pslot * slot_bytes;
+          const int next_col = d_begin + (ci + ahead) * kFCols;
+          const uint32_t next_mask = (ci + ahead < nchunks) ? mask : 0u;  // nothing is fetched past the slice
+          const int next_slot = (pslot == 0) ? ring - 1 : pslot - 1;
+          pslot = (pslot + 1 == ring) ? 0 : pslot + 1;
+          // as in the logit phase: reads, then loads with the MFMAs in between
+          typename Elem<T>::vec8 a[4];
 #pragma unroll
-        for (int ci = 0; ci < kFMaxChunks; ++ci) {
-          if (ci < nchunks) {
-            wait_vmcnt_upto(min(ahead - 1, nchunks - 1 - ci) * 2 * nused);  // the stages after ci may be in flight
-            __syncthreads();
-            const unsigned char* so = smem + pslot * slot_bytes;
-            const int next_col = d_begin + (ci + ahead) * kFCols;
-            const uint32_t next_mask = (ci + ahead < nchunks) ? mask : 0u;  // nothing is fetched past the slice
-            const int next_slot = (pslot == 0) ? ring - 1 : pslot - 1;
-            pslot = (pslot + 1 == ring) ? 0 : pslot + 1;
-            // as in the logit phase: reads, then loads with the MFMAs in between
-            typename Elem<T>::vec8 a[4];
+          for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int j = 0; j < 4; ++j)
+              if ((mask >> ((4 * h + j) >> 1)) & 1u) a[j] = fstage_frag_transposed<T>(so, (4 * h + j) * 16, wave * 32, lane);
 #pragma unroll
-              for (int j = 0; j < 4; ++j)
-                if ((mask >> ((4 * h + j) >> 1)) & 1u) a[j] = fstage_frag_transposed<T>(so, (4 * h + j) * 16, wave * 32, lane);
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                const int kk = 4 * h + j;
-                issue_load(kk, next_col, next_slot, false, next_mask);
-                if ((mask >> (kk >> 1)) & 1u) {
-                  if (ci < 16) Elem<T>::mfma_agpr(a[j], bz[kk], acc[ci]);  // 16 chunks fill the 256 AGPRs
-                  else Elem<T>::mfma_vgpr(a[j], bz[kk], acc[ci]);
-                }
+            for (int j = 0; j < 4; ++j) {
+              const int kk = 4 * h + j;
+              issue_load(kk, next_col, next_slot, false, next_mask);
+              if ((mask >> (kk >> 1)) & 1u) {
+                if constexpr (decltype(in_agpr)::value) Elem<T>::mfma_agpr(a[j], bz[kk], accum);
+                else Elem<T>::mfma_vgpr(a[j], bz[kk], accum);
               }
+            }
+          }
+        };
+        if constexpr (LIGHT) {
+          // one chunk at a time: formed, written straight from the registers (8 bytes per lane and row piece), gone
+#pragma unroll 1
+          for (int ci = 0; ci < nchunks; ++ci) {
+            product_chunk(ci, acc[0], std::false_type{});
+            mfma_drain(acc[0]);
+            store_chunk_direct(ci, acc[0]);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][r] = 0.0f;
+          }
+        } else {
+#pragma unroll
+          for (int ci = 0; ci < kFMaxChunks; ++ci) {
+            if (ci < nchunks) {
+              if (ci < 16) product_chunk(ci, acc[ci], std::true_type{});  // 16 chunks fill the 256 AGPRs
+              else product_chunk(ci, acc[ci], std::false_type{});
             }
           }
         }
@@ -1112,7 +1173,12 @@ __global__ __launch_bounds__(kBwdThreads, 1) void bwd_owner_fast_kernel(BwdParam
 
   mfma_drain_all();  // the last product MFMAs, before anything else reads the accumulators
   const bool out_fp32 = IS_DE ? (p.de_fp32 != 0) : (p.dc_fp32 != 0);
-  if (write_out && (touched || !IS_DE)) {  // dC rows are always written; the launcher guarantees 16-byte aligned rows
+  if constexpr (LIGHT) {
+    if (write_out && !touched) {  // nothing survived for this class group: its rows are zeros
+#pragma unroll 1
+      for (int ci = 0; ci < nchunks; ++ci) store_chunk_direct(ci, acc[0]);
+    }
+  } else if (write_out && (touched || !IS_DE)) {  // dC rows are always written; the launcher guarantees 16-byte aligned rows
     // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
     // are, one instruction would touch 32 rows with 16 bytes each.  Four chunks at a time go through
     // LDS instead and leave as whole rows, 16 bytes per lane and 1 KB per row and instruction.
@@ -1235,10 +1301,13 @@ extern "C" int cce_count_flagged_cells(const float* tile_max, const float* lse, 
 
 static int64_t bit_words_for(int64_t v) { return ((v + 31) / 32 + 31) / 32; }
 
+// survivor bits, then the list of class groups for the full dC pass (a count and up to one id per group)
+static int64_t kept_bits_bytes(int64_t b, int64_t v) { return ((b + 31) / 32) * bit_words_for(v) * 4; }
+
 extern "C" int64_t cce_backward_workspace_bytes(int64_t b, int64_t v, int64_t d) {
   (void)d;
   if (b <= 0 || v <= 0) return 0;
-  return ((b + 31) / 32) * bit_words_for(v) * 4;
+  return kept_bits_bytes(b, v) + (1 + (v + 31) / 32) * 4;
 }
 
 extern "C" int cce_backward(const void* e, const void* c, const void* bias,
@@ -1309,6 +1378,8 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
   p.vec_e = (d_e != nullptr && stride_e % 4 == 0 && d % 4 == 0 && aligned16(d_e)) ? 1 : 0;
   p.vec_c = (d_c != nullptr && stride_cv % 4 == 0 && d % 4 == 0 && stride_cd == 1 && aligned16(d_c)) ? 1 : 0;
   p.sc = make_softcap(softcap);
+  p.light_on = 0;
+  p.heavy_list = nullptr;
 
   // The row-group kernel runs when dE is wanted, and also when only its survivor bits are (dC or
   // dBias filtered); it then skips the products.
@@ -1321,6 +1392,7 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
     if (workspace == nullptr || workspace_bytes < need) return CCE_ERR_WORKSPACE_TOO_SMALL;
     if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return CCE_ERR_MISALIGNED;
     p.kept_bits = static_cast<uint32_t*>(workspace);
+    p.heavy_list = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) + kept_bits_bytes(b, v));
   }
   // Cells may be skipped unseen only if a filtered sub-tile feeds nothing this pass produces.
   p.shortcut = (tile_max != nullptr && vocab_order == nullptr && filtering && filter_eps > 0.0f &&
@@ -1361,6 +1433,31 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
     if (err != hipSuccess) return status_from_hip(err);
   }
   if (need_dc_pass) {
+    // Class groups with at most two surviving entries (most of them when rows are few against the classes) go to a
+    // light variant of the same kernel that holds no gradient in registers and shares a compute unit two by two:
+    // what such a group costs is latency, not work.  It wants a filtered 16-bit dC and one list segment; it
+    // covers all of D itself.  The full variant then skips those groups.
+    const bool light = fast && d_c != nullptr && !d_c_is_fp32 && p.filter_c && p.ntg <= kFListCap;
+    if (light) {
+      BwdParams q = p;
+      q.nslices = 1;
+      q.dslice = static_cast<int>(d);
+      const unsigned grid = static_cast<unsigned>(q.nvg);
+      if (dtype == CCE_DTYPE_BF16) {
+        auto kern = bwd_owner_fast_kernel<BF16, false, true>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kFLightLdsBytes);
+        if (err != hipSuccess) return status_from_hip(err);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kBwdThreads), kFLightLdsBytes, stream, q);
+      } else {
+        auto kern = bwd_owner_fast_kernel<F16, false, true>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kFLightLdsBytes);
+        if (err != hipSuccess) return status_from_hip(err);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kBwdThreads), kFLightLdsBytes, stream, q);
+      }
+      err = hipGetLastError();
+      if (err != hipSuccess) return status_from_hip(err);
+      p.light_on = 1;
+    }
     p.nslices = (d_c != nullptr) ? full_slices : 1;
     const unsigned grid = static_cast<unsigned>(p.nvg) * static_cast<unsigned>(p.nslices);
     CCE_LAUNCH_OWNER(false, grid);

@@ -61,7 +61,8 @@ def test_host_only_queries():
     ws = lib.cce_lse_forward_workspace_bytes(8192, 256000, 2304)
     assert ws > 0 and ws % 8 == 0 and ws <= 16 * 2**20
     # one bit per 32 x 32 sub-tile, rows padded to 32-bit words
-    assert lib.cce_backward_workspace_bytes(8192, 256000, 2304) == 256 * 250 * 4
+    # survivor bits (256 row groups x 250 words) + a count and one id per class group for the second dC pass
+    assert lib.cce_backward_workspace_bytes(8192, 256000, 2304) == 256 * 250 * 4 + (1 + 8000) * 4
     assert lib.cce_backward_workspace_bytes(0, 5, 5) == 0
 
 
