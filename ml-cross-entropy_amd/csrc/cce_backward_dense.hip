@@ -83,20 +83,18 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
   s.b_row[0] = nullptr;
   s.a_km = nullptr;
   s.a_stride = 0;
-  s.a_ok = true;
-  const int bcol = n0 + Tile::chunk_kmajor(g.wave, g.lane);
-  s.b_km = p.c + bcol;
-  s.b_ok = bcol < p.d;
+  // (columns past d: the last chunk inside the matrix once more; what they feed is dropped below)
+  s.b_km = p.c + min(n0 + Tile::chunk_kmajor(g.wave, g.lane), p.d - 8);
   s.b_stride = p.stride_cv;
   s.b_rows = nullptr;
   s.k_total = p.n_cls;
-  s.k_last = ((p.n_cls + Tile::BK - 1) / Tile::BK - 1) * Tile::BK;
 
   f32x16 acc[Tile::WM][Tile::WN];
-  int ids[Tile::NQ1];
+  typename Tile::Loop loop = Tile::plan(s, g);
+  typename Tile::Ids ids;
   typename Tile::Ptrs ptrs;
-  Tile::prefetch(s, ptrs, ids, g);
-  Tile::run(acc, s, ptrs, ids, smem, g);
+  Tile::prefetch(s, loop, ptrs, ids, g);
+  Tile::run(acc, s, loop, ptrs, ids, smem, g);
 
   Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
     const int64_t ri = m0 + row;          // valid-row number
@@ -140,10 +138,10 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
   });
 }
 
-// dC[class][col] = sum_row dz[row][class] * E[row][col]
-template <typename T>
+// dC[class][col] = sum_row dz[row][class] * E[row][col]; GATHER: the rows of E come through valids
+template <typename T, bool GATHER>
 __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, int tn, unsigned char* smem) {
-  using Tile = Tile4<T, true, true>;
+  using Tile = Tile4<T, true, true, GATHER>;
   typename Tile::Geometry g = Tile::geometry(smem);
   const int m0 = tm * Tile::TILE;
   const int n0 = tn * Tile::TILE;
@@ -152,21 +150,20 @@ __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, in
   s.a_row[0] = nullptr;
   s.b_row[0] = nullptr;
   const int chunk = Tile::chunk_kmajor(g.wave, g.lane);
-  s.a_km = p.dz + m0 + chunk;
-  s.a_ok = (m0 + chunk) < p.ldz;
+  // (columns past the matrix: the last chunk inside it once more; what they feed is dropped below)
+  s.a_km = p.dz + min(static_cast<int64_t>(m0 + chunk), p.ldz - 8);
   s.a_stride = p.ldz;
-  s.b_km = p.e + n0 + chunk;
-  s.b_ok = (n0 + chunk) < p.d;
+  s.b_km = p.e + min(n0 + chunk, p.d - 8);
   s.b_stride = p.stride_e;
   s.b_rows = p.valids;
   s.k_total = static_cast<int>(p.b);
-  s.k_last = 0;
 
   f32x16 acc[Tile::WM][Tile::WN];
-  int ids[Tile::NQ1];
+  typename Tile::Loop loop = Tile::plan(s, g);
+  typename Tile::Ids ids;
   typename Tile::Ptrs ptrs;
-  Tile::prefetch(s, ptrs, ids, g);
-  Tile::run(acc, s, ptrs, ids, smem, g);
+  Tile::prefetch(s, loop, ptrs, ids, g);
+  Tile::run(acc, s, loop, ptrs, ids, smem, g);
 
   Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
     const int cls = m0 + row;
@@ -202,7 +199,11 @@ __global__ __launch_bounds__(kProdThreads, 1) void dense_products_kernel(Product
   int tm, tn;
   if (first != (p.de_first != 0)) {
     if (!product_tile_of(block, p.dc_tiles, p.dc_per_xcd, p.tiles_n, tm, tn)) return;
-    dense_dc_tile<T>(p, tm, tn, smem);
+    if (p.valids != nullptr) {
+      dense_dc_tile<T, true>(p, tm, tn, smem);
+    } else {
+      dense_dc_tile<T, false>(p, tm, tn, smem);
+    }
   } else {
     if (!product_tile_of(block, p.de_tiles, p.de_per_xcd, p.tiles_n, tm, tn)) return;
     dense_de_tile<T, SPLIT_DE>(p, tm, tn, smem);
