@@ -3,8 +3,9 @@
 // written to memory in the input type (or as fp32), for the unfiltered ("exact") backward: with every entry of
 // the gradient in play the two products dE = dz . C and dC = dz^T . E are dense matrix products over the chunk,
 // which the kernels of cce_backward_dense.hip run.  The kernel is the forward kernel with another epilogue: same work
-// items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as whole rows
-// of 256 bytes per wave instruction after a transposition through LDS.
+// items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as row pieces of 128
+// contiguous bytes (8 rows per wave instruction) after a transposition through LDS, while the first stages of the
+// next tile are already arriving.
 #include "cce_dense.h"
 
 namespace cce {
@@ -34,15 +35,15 @@ struct DzParams {
 constexpr int kDzWV = 4, kDzWT = 2, kDzNWV = 2, kDzNWT = 4;  // the forward kernel's wave tiling
 constexpr int kDzThreads = 64 * kDzNWV * kDzNWT;
 constexpr int kDzTile = 256;
-constexpr int kDzStagePitch = 128 * 2 + 16;  // one row of a wave's staged block (128 x 16-bit or 64 x fp32), padded
-constexpr int kDzStageBytes = 32 * kDzStagePitch;
+constexpr int kDzStageRow = 128;                  // bytes of one row of a wave's staged block (64 x 16-bit or 32 x fp32)
+constexpr int kDzStageBytes = 32 * kDzStageRow;   // 32 rows
 
 // OUT32: dz leaves as fp32 (for inputs that are fp32 values split into 16-bit parts along D, whose
-// gradients are wanted at fp32 accuracy): a staged block is then 32 rows x 64 classes.
+// gradients are wanted at fp32 accuracy): a staged block is then 32 rows x 32 classes.
 template <typename T, bool GENERAL, bool OUT32>
 __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
   using Fast = DmaLogitTile<T, kDzWV, kDzWT, kDzNWV, kDzNWT>;
-  static_assert(kDzStageBytes * kDzNWV * kDzNWT <= Fast::LDS_BYTES, "the staging blocks reuse the idle ring");
+  static_assert(kDzStageBytes * kDzNWV * kDzNWT <= Fast::TILE_T * kDmaRowBytes, "the staging blocks fit the token half of a stage");
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_addend = reinterpret_cast<float*>(smem + Fast::LDS_BYTES);  // [2][256]
 
@@ -99,19 +100,27 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
     r_tgt[ti] = tgt;
   }
 
-  unsigned char* stage = smem + wave * kDzStageBytes;
+  // Staged blocks live in the token half of LDS stage 1, the one part of the ring that the early fetch of the
+  // next tile (all of stage 0, the class half of stage 1) leaves alone.
+  unsigned char* stage = smem + Fast::STAGE_BYTES + Fast::TILE_V * kDmaRowBytes + wave * kDzStageBytes;
 
-  for (int vt = vt_begin; vt < vt_end; ++vt) {
+  auto point_at_tile = [&](int vt) {
     const int64_t v0 = static_cast<int64_t>(vt) * kDzTile;
-    float* addend = s_addend + (vt & 1) * kDzTile;
-    __syncthreads();  // every wave has left the staging blocks of the previous tile: the ring may be refilled
 #pragma unroll
     for (int q = 0; q < Fast::NQC; ++q) {
       int64_t vr = v0 + Fast::row_of(q, wave, lane);
       vr = (vr < p.v) ? vr : p.v - 1;  // classes past the end repeat the last one; masked below
       fptr[q] = p.c + vr * p.stride_cv + Fast::chunk_elems(wave, lane);
     }
+  };
+  if (vt_begin < vt_end) {
+    point_at_tile(vt_begin);
     Fast::prefetch(fptr, smem, static_cast<int>(p.d));
+  }
+
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int64_t v0 = static_cast<int64_t>(vt) * kDzTile;
+    float* addend = s_addend + (vt & 1) * kDzTile;
     if (GENERAL) {
       if (tid < kDzTile) {  // published by the barriers of the main loop
         const int64_t vg = v0 + tid;
@@ -121,20 +130,28 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
       }
     }
     f32x16 acc[kDzWV][kDzWT];
-    Fast::run(acc, fptr, smem, static_cast<int>(p.d));
+    Fast::run(acc, fptr, smem, static_cast<int>(p.d));  // (ends with a barrier: the ring is idle)
+    // The next tile starts to arrive while this one's gradients are formed and stored.  Its loads sit ahead of the
+    // stores below in the queue the main loop counts by: loads complete in order among themselves, so "at most QA
+    // operations outstanding" at the top of run() still means that stage 0 has landed.
+    if (vt + 1 < vt_end) {
+      point_at_tile(vt + 1);
+      Fast::prefetch(fptr, smem, static_cast<int>(p.d));
+    }
 
     const int cls0 = static_cast<int>(v0) + wv * (32 * kDzWV);  // first class of this wave
     const float* wave_addend = addend + wv * (32 * kDzWV);
+    const int sw = (l32 >> 1) & 7;  // 16-byte chunks of a staged row are XOR-swizzled with (row >> 1) & 7
 #pragma unroll
     for (int ti = 0; ti < kDzWT; ++ti) {
       const float lse2 = r_lse2[ti], g = r_g[ti], gh = r_g[ti] + r_h[ti];
       const int tgt = r_tgt[ti];
-      constexpr int kHalves = OUT32 ? 2 : 1;        // staged blocks per column block
-      constexpr int kViPer = kDzWV / kHalves;       // 32-class blocks per staged block
-      constexpr int kEs = OUT32 ? 4 : 2;            // bytes per stored element
-      constexpr int kPieceElems = 16 / kEs;         // elements per 16-byte piece
+      constexpr int kEs = OUT32 ? 4 : 2;                    // bytes per stored element
+      constexpr int kViPer = kDzStageRow / (32 * kEs);      // 32-class blocks per staged block (2, or 1 for fp32)
+      constexpr int kParts = kDzWV / kViPer;                // staged blocks per column block
+      constexpr int kPieceElems = 16 / kEs;                 // elements per 16-byte piece
 #pragma unroll
-      for (int vh = 0; vh < kHalves; ++vh) {
+      for (int vh = 0; vh < kParts; ++vh) {
 #pragma unroll
         for (int vj = 0; vj < kViPer; ++vj) {
           const int vi = vh * kViPer + vj;
@@ -166,7 +183,8 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
               dz *= damp;
               dzv[i] = dead ? 0.0f : dz;
             }
-            unsigned char* dst = stage + l32 * kDzStagePitch + (vj * 32 + 8 * r4 + 4 * half) * kEs;
+            const int col = (vj * 32 + 8 * r4 + 4 * half) * kEs;  // byte inside the staged row
+            unsigned char* dst = stage + l32 * kDzStageRow + ((((col >> 4) ^ sw) << 4) | (col & 15));
             if (OUT32) {
               *reinterpret_cast<float4*>(dst) = make_float4(dzv[0], dzv[1], dzv[2], dzv[3]);
             } else {
@@ -178,13 +196,13 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
           }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is private to this wave: no barrier
-        // 32 rows x 256 bytes leave as 16-byte pieces: one instruction covers 4 rows of 256 contiguous bytes
+        // 32 rows x 128 bytes leave as 16-byte pieces: one instruction covers 8 rows of 128 contiguous bytes
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < 4; ++k) {
           const int j = lane + 64 * k;
-          const int row = j >> 4;
-          const int pc = j & 15;
-          const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kDzStagePitch + pc * 16);
+          const int row = j >> 3;
+          const int pc = j & 7;
+          const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kDzStageRow + ((pc ^ ((row >> 1) & 7)) << 4));
           const int64_t gi = t0 + wt * (32 * kDzWT) + ti * 32 + row;
           const int64_t gcol = static_cast<int64_t>(cls0) + vh * (32 * kViPer) + pc * kPieceElems;
           if (gi < p.b) {
