@@ -14,9 +14,9 @@ from cut_cross_entropy.utils import TensorInfo
 # Upper bound of the dz chunk buffer of the unfiltered backward (bytes).  The chunk is [B, vc] in the input type
 # with vc a multiple of 256 classes, at most 16384; the library picks the vc that fits and fills the 256 compute
 # units most evenly.  A smaller buffer means more, smaller chunks: less memory, more launches and more passes over
-# the dE accumulator (measured, backward of E [15356, 4096] x C [128256, 4096]: 44.4 ms with 128 MB, 41.0 with
-# 256; E [8192, 2048] x C [256000, 2048]: 21.8 / 21.8; E [8192, 2304] x C [256000, 2304]: 24.8 / 25.7; with 32 MB
-# the last one takes 31.8).  On top of it comes, when dE is wanted in a 16-bit type, a [B, D] 16-bit
+# the dE accumulator (measured, backward of E [15356, 4096] x C [128256, 4096]: 44.1 ms with 128 MB, 40.4 with
+# 256; E [8192, 2048] x C [256000, 2048]: 21.5 / 21.5; E [8192, 2304] x C [256000, 2304]: 24.4 / 24.0; with 32 MB
+# the last one takes 29.7).  On top of it comes, when dE is wanted in a 16-bit type, a [B, D] 16-bit
 # compensation buffer (dE is summed over the chunks as a pair of 16-bit numbers).
 DENSE_DZ_BYTES = 256 << 20
 
