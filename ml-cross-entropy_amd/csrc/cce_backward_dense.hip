@@ -54,14 +54,37 @@ struct ProductParams {
 
 constexpr int kProdThreads = 256;  // four waves, one per SIMD
 
-// Tile `block` of a group of `tiles` tiles: ids that land on one XCD get consecutive tiles, which share the A operand.
+// Tile `block` of a group of `tiles` tiles (tiles_n column tiles wide).  Block ids that land on one XCD get
+// consecutive places in an order that keeps the 32 tiles an XCD works on at a time on few operand panels: a tile
+// streams one A panel (its row of tiles) and one B panel (its column) through the XCD's L2, so 32 tiles of one or
+// two rows of a wide output need 2 + 16 panels where a block of 4 x 8 tiles needs 12.  The columns are therefore
+// cut into groups of at most 8 (as equal as possible), and the order walks a group row by row before it moves to
+// the next group (E [15356, 4096] x C [128256, 4096], 16 column tiles: backward 39.3 -> 38.1 ms).
 __device__ __forceinline__ bool product_tile_of(int block, int tiles, int per_xcd, int tiles_n, int& tm, int& tn) {
   const int xcd = block & 7;
   const int slot = block >> 3;
-  const int lin = xcd * per_xcd + slot;
+  int lin = xcd * per_xcd + slot;
   if (lin >= tiles) return false;
-  tm = lin / tiles_n;
-  tn = lin - tm * tiles_n;
+  const int tiles_m = tiles / tiles_n;
+  const int groups = (tiles_n + 7) / 8;
+  const int narrow = tiles_n / groups;          // width of the narrow groups; the first `wide` groups have one more
+  const int wide = tiles_n - narrow * groups;
+  const int in_wide = wide * tiles_m * (narrow + 1);
+  int width, first_col;
+  if (lin < in_wide) {
+    width = narrow + 1;
+    const int grp = lin / (tiles_m * width);
+    lin -= grp * tiles_m * width;
+    first_col = grp * width;
+  } else {
+    width = narrow;
+    lin -= in_wide;
+    const int grp = lin / (tiles_m * width);
+    lin -= grp * tiles_m * width;
+    first_col = wide * (narrow + 1) + grp * width;
+  }
+  tm = lin / width;
+  tn = first_col + (lin - tm * width);
   return true;
 }
 
