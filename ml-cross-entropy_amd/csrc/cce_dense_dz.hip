@@ -6,6 +6,8 @@
 // items, same direct-to-LDS main loop, logits never leave the registers; only dz does, as row pieces of 128
 // contiguous bytes (8 rows per wave instruction) after a transposition through LDS, while the first stages of the
 // next tile are already arriving.
+#include <type_traits>
+
 #include "cce_dense.h"
 
 namespace cce {
@@ -152,48 +154,57 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz_kernel(DzParams p) {
       constexpr int kPieceElems = 16 / kEs;                 // elements per 16-byte piece
 #pragma unroll
       for (int vh = 0; vh < kParts; ++vh) {
+        // The gradients of one staged block.  One copy of the arithmetic per answer to "soft-capped?": asked per
+        // logit, the (uniform) question costs two branches per element, a third of the epilogue's time.
+        auto stage_block = [&](auto capped) {
 #pragma unroll
-        for (int vj = 0; vj < kViPer; ++vj) {
-          const int vi = vh * kViPer + vj;
+          for (int vj = 0; vj < kViPer; ++vj) {
+            const int vi = vh * kViPer + vj;
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            float dzv[4];
+            for (int r4 = 0; r4 < 4; ++r4) {
+              float dzv[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int cl = vi * 32 + 8 * r4 + 4 * half + i;
-              float x = acc[vi][ti][r4 * 4 + i];
-              bool dead = false;
-              if (GENERAL) {
-                const float add = wave_addend[cl];
-                dead = (add == -INFINITY);
-                x = dead ? 0.0f : x + add;
+              for (int i = 0; i < 4; ++i) {
+                const int cl = vi * 32 + 8 * r4 + 4 * half + i;
+                float x = acc[vi][ti][r4 * 4 + i];
+                bool dead = false;
+                if (GENERAL) {
+                  const float add = wave_addend[cl];
+                  dead = (add == -INFINITY);
+                  x = dead ? 0.0f : x + add;
+                }
+                float s2, damp = 1.0f;
+                if (decltype(capped)::value) {
+                  const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
+                  const float w = __builtin_amdgcn_rcpf(1.0f + t);
+                  const float th = 1.0f - 2.0f * w;
+                  s2 = p.sc.out_scale * th;
+                  damp = 1.0f - th * th;
+                } else {
+                  s2 = x * kLog2e;
+                }
+                const float pr = __builtin_amdgcn_exp2f(s2 - lse2);
+                float dz = pr * gh - ((cls0 + cl == tgt) ? g : 0.0f);
+                if (decltype(capped)::value) dz *= damp;
+                dzv[i] = dead ? 0.0f : dz;
               }
-              float s2, damp = 1.0f;
-              if (p.sc.on) {
-                const float t = __builtin_amdgcn_exp2f(x * p.sc.in_scale);
-                const float w = __builtin_amdgcn_rcpf(1.0f + t);
-                const float th = 1.0f - 2.0f * w;
-                s2 = p.sc.out_scale * th;
-                damp = 1.0f - th * th;
+              const int col = (vj * 32 + 8 * r4 + 4 * half) * kEs;  // byte inside the staged row
+              unsigned char* dst = stage + l32 * kDzStageRow + ((((col >> 4) ^ sw) << 4) | (col & 15));
+              if (OUT32) {
+                *reinterpret_cast<float4*>(dst) = make_float4(dzv[0], dzv[1], dzv[2], dzv[3]);
               } else {
-                s2 = x * kLog2e;
+                uint2 pk;
+                pk.x = Elem<T>::pack2(dzv[0], dzv[1]);
+                pk.y = Elem<T>::pack2(dzv[2], dzv[3]);
+                *reinterpret_cast<uint2*>(dst) = pk;
               }
-              const float pr = __builtin_amdgcn_exp2f(s2 - lse2);
-              float dz = pr * gh - ((cls0 + cl == tgt) ? g : 0.0f);
-              dz *= damp;
-              dzv[i] = dead ? 0.0f : dz;
-            }
-            const int col = (vj * 32 + 8 * r4 + 4 * half) * kEs;  // byte inside the staged row
-            unsigned char* dst = stage + l32 * kDzStageRow + ((((col >> 4) ^ sw) << 4) | (col & 15));
-            if (OUT32) {
-              *reinterpret_cast<float4*>(dst) = make_float4(dzv[0], dzv[1], dzv[2], dzv[3]);
-            } else {
-              uint2 pk;
-              pk.x = Elem<T>::pack2(dzv[0], dzv[1]);
-              pk.y = Elem<T>::pack2(dzv[2], dzv[3]);
-              *reinterpret_cast<uint2*>(dst) = pk;
             }
           }
+        };
+        if (p.sc.on) {
+          stage_block(std::true_type{});
+        } else {
+          stage_block(std::false_type{});
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is private to this wave: no barrier
         // 32 rows x 128 bytes leave as 16-byte pieces: one instruction covers 8 rows of 128 contiguous bytes
