@@ -112,6 +112,30 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
   s.b_rows = nullptr;
   s.k_total = p.n_cls;
 
+  // What memory holds of a piece so far, fetched ahead of its use.
+  struct Old {
+    int64_t re;   // the piece's row of e (-1: the piece lies outside the matrix)
+    uint4 a, b;   // fp32 dE: the eight sums; a 16-bit dE: the hi and the lo halves of the eight sums
+  };
+  auto fetch = [&](int row, int col) {
+    Old o;
+    o.re = -1;
+    o.a = make_uint4(0u, 0u, 0u, 0u);
+    o.b = make_uint4(0u, 0u, 0u, 0u);
+    const int64_t ri = m0 + row;          // valid-row number
+    const int cg = n0 + col;
+    if (ri >= p.b || cg >= p.d) return o;
+    o.re = (p.valids != nullptr && !p.de_rows_by_number) ? static_cast<int64_t>(p.valids[ri]) : ri;
+    if (!SPLIT_DE) {
+      const uint4* src = reinterpret_cast<const uint4*>(p.de_f32 + o.re * p.ld_de + cg);
+      o.a = src[0];
+      o.b = src[1];
+    } else if (!p.first_chunk) {
+      o.a = *reinterpret_cast<const uint4*>(p.de_hi + o.re * p.ld_de + cg);
+      o.b = *reinterpret_cast<const uint4*>(p.de_lo + ri * p.d + cg);
+    }
+    return o;
+  };
   f32x16 acc[Tile::WM][Tile::WN];
   typename Tile::Loop loop = Tile::plan(s, g);
   typename Tile::Ids ids;
@@ -119,14 +143,16 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
   Tile::prefetch(s, loop, ptrs, ids, g);
   Tile::run(acc, s, loop, ptrs, ids, smem, g);
 
-  Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
-    const int64_t ri = m0 + row;          // valid-row number
+  // (fetching the first slabs before the main loop instead would hold 80 registers across it: they spill)
+  typename Tile::template Rmw<Old> rmw;
+  Tile::rmw_begin(rmw, g, fetch);
+  Tile::for_each_row_piece_rmw(acc, smem, g, rmw, fetch, [&](int row, int col, const float (&v)[8], const Old& o) {
+    if (o.re < 0) return;
+    const int64_t ri = m0 + row;
     const int cg = n0 + col;
-    if (ri >= p.b || cg >= p.d) return;
-    const int64_t re = (p.valids != nullptr && !p.de_rows_by_number) ? static_cast<int64_t>(p.valids[ri]) : ri;  // its row of e
     if (!SPLIT_DE) {
-      float4* dst = reinterpret_cast<float4*>(p.de_f32 + re * p.ld_de + cg);
-      float4 a = dst[0], b = dst[1];
+      float4* dst = reinterpret_cast<float4*>(p.de_f32 + o.re * p.ld_de + cg);
+      float4 a = __builtin_bit_cast(float4, o.a), b = __builtin_bit_cast(float4, o.b);
       a.x += v[0]; a.y += v[1]; a.z += v[2]; a.w += v[3];
       b.x += v[4]; b.y += v[5]; b.z += v[6]; b.w += v[7];
       dst[0] = a;
@@ -134,14 +160,9 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
     } else {
       // value so far = hi + lo (two 16-bit numbers: 16 bits of mantissa, where one would round the sum of a few
       // dozen chunks eight bits short); the new hi is the rounded total, so the last chunk leaves d_e final
-      uint4* hi_ptr = reinterpret_cast<uint4*>(p.de_hi + re * p.ld_de + cg);
+      uint4* hi_ptr = reinterpret_cast<uint4*>(p.de_hi + o.re * p.ld_de + cg);
       uint4* lo_ptr = reinterpret_cast<uint4*>(p.de_lo + ri * p.d + cg);
-      uint4 hi = make_uint4(0u, 0u, 0u, 0u), lo = make_uint4(0u, 0u, 0u, 0u);
-      if (!p.first_chunk) {
-        hi = *hi_ptr;
-        lo = *lo_ptr;
-      }
-      const uint32_t hw[4] = {hi.x, hi.y, hi.z, hi.w}, lw[4] = {lo.x, lo.y, lo.z, lo.w};
+      const uint32_t hw[4] = {o.a.x, o.a.y, o.a.z, o.a.w}, lw[4] = {o.b.x, o.b.y, o.b.z, o.b.w};
       uint32_t ho[4], lo_out[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {

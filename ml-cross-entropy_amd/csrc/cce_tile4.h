@@ -461,6 +461,60 @@ struct Tile4 {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the next slab is staged
     });
   }
+
+  // The same for an output that is combined with what memory holds (dE is summed over the chunks): `fetch(row,
+  // col)` returns what `store(row, col, v, old)` needs of the old contents.  The fetches of a slab are issued two
+  // slabs ahead (a slab takes about a microsecond, a load under this traffic up to two, two dependent ones where
+  // the rows are gathered), those of the first two slabs by rmw_begin() right before, so that their latency is paid
+  // once per tile and not once per slab.
+  static constexpr int kSlabs = WM * (WN / 2);
+  static constexpr int kAhead = 2;
+  template <typename Old>
+  struct Rmw {
+    Old old[kAhead + 1][4];
+  };
+  template <int SLAB, typename Old, typename Fetch>
+  static __device__ __forceinline__ void rmw_fetch(Rmw<Old>& r, const Geometry& g, Fetch&& fetch) {
+    constexpr int i = SLAB / (WN / 2);
+    constexpr int jp = SLAB % (WN / 2);
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass)
+      r.old[SLAB % (kAhead + 1)][pass] =
+          fetch(g.wm * 128 + i * 32 + pass * 8 + (g.lane >> 3), g.wn * 128 + jp * 64 + (g.lane & 7) * kPieceCols);
+  }
+  template <typename Old, typename Fetch>
+  static __device__ __forceinline__ void rmw_begin(Rmw<Old>& r, const Geometry& g, Fetch&& fetch) {
+    static_for<kAhead>([&](auto slab) { rmw_fetch<decltype(slab)::value>(r, g, fetch); });
+  }
+  template <typename Old, typename Fetch, typename Store>
+  static __device__ __forceinline__ void for_each_row_piece_rmw(f32x16 (&acc)[WM][WN], unsigned char* lds, const Geometry& g,
+                                                                Rmw<Old>& r, Fetch&& fetch, Store&& store) {
+    unsigned char* stage = lds + g.wave * kStageBytes;
+    const int c8 = (g.lane & 7) * kPieceCols;
+    const int m_lane = g.lane >> 3;
+    static_for<kSlabs>([&](auto ij) {
+      constexpr int i = decltype(ij)::value / (WN / 2);
+      constexpr int jp = decltype(ij)::value % (WN / 2);
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int rr = 0; rr < 16; ++rr) {
+          const int m = 8 * (rr >> 2) + 4 * g.half + (rr & 3);
+          *reinterpret_cast<float*>(stage + m * kStagePitch + (jj * 32 + g.l32) * 4) = acc[i][jp * 2 + jj][rr];
+        }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if constexpr (decltype(ij)::value + kAhead < kSlabs) rmw_fetch<decltype(ij)::value + kAhead>(r, g, fetch);
+#pragma unroll
+      for (int pass = 0; pass < 4; ++pass) {
+        const int m = pass * 8 + m_lane;
+        const float4 lo = *reinterpret_cast<const float4*>(stage + m * kStagePitch + c8 * 4);
+        const float4 hi = *reinterpret_cast<const float4*>(stage + m * kStagePitch + c8 * 4 + 16);
+        const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        store(g.wm * 128 + i * 32 + m, g.wn * 128 + jp * 64 + c8, v, r.old[decltype(ij)::value % (kAhead + 1)][pass]);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the next slab is staged
+    });
+  }
 };
 
 }  // namespace cce

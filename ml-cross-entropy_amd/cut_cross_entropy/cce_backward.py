@@ -20,6 +20,16 @@ from cut_cross_entropy.utils import TensorInfo
 # compensation buffer (dE is summed over the chunks as a pair of 16-bit numbers).
 DENSE_DZ_BYTES = 256 << 20
 
+# ... but never so small that a chunk holds fewer classes than this: with many rows (B = 65536: 2048 classes in
+# 256 MB) the tiles of dE have a short reduction, their fetch and read-modify-write of dE weigh as much as their
+# products, and dE is passed over once per chunk (measured, backward of E [65536, 3584] x C [19008, 3584]: 24.9 ms
+# with 256 MB, 21.7 with 512, 21.1 with 1024).  The buffer then grows with B like E and dE themselves do.
+DENSE_DZ_MIN_CLASSES = 4096
+
+
+def _dz_budget(B: int) -> int:
+    return max(int(DENSE_DZ_BYTES), 2 * int(B) * int(DENSE_DZ_MIN_CLASSES))
+
 # With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path pays for
 # the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
 # statistic can hold a probability above filter_eps for E [8192, 2304] x C [256000, 2304], and at 0.083 for
@@ -82,7 +92,7 @@ def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, fi
     if DENSE_WHEN_FLAGGED_ABOVE is None:
         return False
     if (DENSE_WORKSPACE_LIMIT_BYTES is not None
-            and lib.cce_backward_dense_workspace_bytes(B, V, D, 1, DENSE_DZ_BYTES) > DENSE_WORKSPACE_LIMIT_BYTES):
+            and lib.cce_backward_dense_workspace_bytes(B, V, D, 1, _dz_budget(B)) > DENSE_WORKSPACE_LIMIT_BYTES):
         return False
     key = (dev.index, V, D, dtype)
     with _monitors_lock:
@@ -121,7 +131,7 @@ def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, 
     allocator's peak statistic sees it."""
     V, D = c.size(0), e.size(1)
     de_in_ws = de is not None and de.dtype != torch.float32
-    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_in_ws else 0, DENSE_DZ_BYTES)
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_in_ws else 0, _dz_budget(B))
     workspace = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
     ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
     with torch.cuda.device(dev), _hip.timed("backward_dense", dev):
