@@ -377,10 +377,13 @@ def test_entry_points_reject_bad_arguments_before_launching():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(256, 512, 128), (300, 500, 72), (1000, 130, 264), (33, 64, 8)])
+@pytest.mark.parametrize("shape", [(256, 512, 128), (300, 500, 72), (1000, 130, 264), (33, 64, 8),
+                                   (63, 40, 64), (65, 257, 520), (1, 7, 8), (130, 64, 1032)])
 def test_backward_products_abi(dtype, shape):
     """cce_backward_products: d_e += dz . c and d_c (+)= dz^T . e[valids] with fp32 results, against the same
-    products in fp64 of the same 16-bit inputs (exact up to fp32 accumulation: 1e-5 of the row scale)."""
+    products in fp64 of the same 16-bit inputs (exact up to fp32 accumulation: 1e-5 of the row scale).  Among
+    the shapes: reductions shorter than one 64-step stage (no whole stage: the main loop only fetches zeros), one
+    step longer than a stage (the partial stage goes first), five column tiles (two groups in the tile order)."""
     lib = _lib()
     dev = torch.device("cuda:0")
     B, M, D = shape
