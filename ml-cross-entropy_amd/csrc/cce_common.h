@@ -19,6 +19,7 @@
 namespace cce {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -55,6 +56,11 @@ struct Elem<BF16> {
   }
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  // 16 x 16 block, 32 reduction elements: lane l holds row (l % 16), elements 8 (l / 16) .. + 7 of either operand
+  // and, of the result, column (l % 16), rows 4 (l / 16) + r, r = 0 .. 3.
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
   // The same MFMA with the accumulator pinned to one register file: "a" = the accumulation registers
   // (AGPRs), "v" = the ordinary ones.  For kernels whose accumulators outnumber the 256 AGPRs: the
@@ -97,6 +103,9 @@ struct Elem<F16> {
   }
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ void mfma_agpr(vec8 a, vec8 b, f32x16& c) {
     asm volatile("s_nop 4\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 11" : "+a"(c) : "v"(a), "v"(b));
@@ -299,6 +308,12 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr)
                : "memory", "m0");
 }
+// The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit byte offset per
+// lane: half the vector registers per address, and what changes from stage to stage is added on the scalar unit.
+__device__ __forceinline__ void lds_dma16_sbase(const void* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 
 template <typename F, int... Is>
@@ -479,6 +494,184 @@ struct DmaLogitTile {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unused prefetch
     __syncthreads();  // every wave is done with the LDS (the last prefetch was awaited above)
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// The same logit tile from 16 x 16 x 32 MFMAs.  The matrix pipes of this chip are limited by power, not by
+// issue: with operands of full entropy the 32 x 32 x 16 instruction sustains 1.84 PFLOP/s from registers alone
+// and the 16 x 16 x 32 one 2.09 (it reads and writes a quarter of the accumulator registers per instruction and
+// adds twice as many products before it touches them), both 2.46 with operands of zeros; the clock the chip holds
+// under the forward kernel rises accordingly.  Same tile, ring and loads as DmaLogitTile; what changes is who
+// holds what:
+//   wave (wv, wt) owns WV x WT blocks of 16 classes x 16 token rows; lane l holds, of every block, the token row
+//   (l % 16) and the classes 4 (l / 16) + r, r = 0 .. 3; a fragment is 16 rows x 32 reduction columns = half a
+//   ring row, lane l reads 16-byte chunk (l / 16) (+ 4 for the second half) of row (l % 16): one fragment read is
+//   four groups of 16 rows x one chunk, each covering all 64 banks through the XOR swizzle.
+// Pipeline, per 64-column stage two steps of WV x WT MFMAs: the step on columns 0 .. 31 reads the fragments of
+// columns 32 .. 63 of the same stage, the step on columns 32 .. 63 those of the next stage's first half and
+// issues ALL loads of the stage after that into the ring stage it has just finished with.  A class fragment
+// is re-read in place as soon as its WT MFMAs are issued (so only the token fragments are held twice); one
+// barrier per stage, a few MFMAs into the second step, at which the loads issued most of a stage earlier have landed.
+// The stages run on across the tiles of a span: the loads issued under the last two stages of a tile fetch the
+// first two stages of the NEXT tile (next_tile() swaps the class pointers), so that nothing is fetched that is
+// not consumed and the next main loop starts with its data in LDS, whatever the epilogue in between does.
+// `buf` carries the ring stage the next tile starts in (it alternates when D / 64 is odd).
+// ---------------------------------------------------------------------------------------------
+template <typename T, int WV, int WT, int NWV, int NWT>
+struct DmaLogitTile16 {
+  static_assert(WV % 2 == 0 && WT % 2 == 0, "the ring is addressed in blocks of 32 rows");
+  using Base = DmaLogitTile<T, WV / 2, WT / 2, NWV, NWT>;
+  static constexpr int TILE_V = Base::TILE_V;
+  static constexpr int TILE_T = Base::TILE_T;
+  static constexpr int NW = Base::NW;
+  static constexpr int STAGE_BYTES = Base::STAGE_BYTES;
+  static constexpr int LDS_BYTES = Base::LDS_BYTES;
+  static constexpr int NQC = Base::NQC;
+  static constexpr int NQ = Base::NQ;
+  using vec8 = typename Elem<T>::vec8;
+
+  static __device__ __forceinline__ int row_of(int q, int wave, int lane) { return Base::row_of(q, wave, lane); }
+  static __device__ __forceinline__ int chunk_elems(int wave, int lane) { return Base::chunk_elems(wave, lane); }
+
+  // Where the loads of a tile come from: per load a 32-bit byte offset of this lane's row and chunk, relative to a
+  // wave-uniform base -- the first class row of the tile for the class loads, the matrix of token rows for the others.
+  struct Source {
+    unsigned off[NQ];
+    const unsigned char* c_base;
+    const unsigned char* e_base;
+  };
+
+  static __device__ __forceinline__ vec8 frag(const unsigned char* p) {
+    return __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(p));
+  }
+
+  // Load q of one stage, columns [k0, k0 + 64), into ring stage `stage_off`.
+  static __device__ __forceinline__ void issue_one(const Source& src, int q, int k0, unsigned lds_base, int stage_off,
+                                                   int wave) {
+    const int blk = (q < NQC) ? (q * NW + wave) : (TILE_V / 8 + (q - NQC) * NW + wave);
+    const unsigned char* base = ((q < NQC) ? src.c_base : src.e_base) + 2 * k0;
+    lds_dma16_sbase(base, src.off[q], lds_base + stage_off + blk * 1024);
+  }
+
+  // One step: WV x WT MFMAs on the class fragments a[] and the token fragments bc[]; under them, at most one
+  // memory instruction after each MFMA:
+  //   READ  the fragments of the next step from rd_c / rd_e (ring stage + this lane's chunk): class fragment vi
+  //         into a[vi] once the last MFMA that uses the old one is issued, the token fragments into bn[];
+  //   LOAD  all loads of a later stage (columns koff ..) into ring stage `ld_stage`.
+  // SYNC (the step on the second half of a stage): after the first WT MFMAs, which need nothing new, this wave
+  // waits for its own loads of the next stage and for the fragment reads it still has in flight, then the
+  // barrier: from there on the next stage may be read and the stage this step computes on (every wave holds
+  // its last fragments of it) may be overwritten.  Reads and loads of such a step all come after the barrier.
+  // (With the barrier between the steps instead, every wave met it with its last fragment read just issued and
+  // the compute units idled a sixth of the time.)
+  static constexpr int kSyncAt = WT;  // MFMAs of a SYNC step issued before the barrier
+  static constexpr int kSlots = WV * WT;
+  static constexpr int a_slot(bool sync, int vi) {
+    const int natural = vi * WT + WT - 1;  // the last MFMA that reads a[vi]
+    return (sync && natural < kSyncAt + 1 + 2 * vi) ? kSyncAt + 1 + 2 * vi : natural;
+  }
+  static constexpr int b_slot(bool sync, int t) {
+    return sync ? kSyncAt + 5 + t * ((kSlots - kSyncAt - 8) / WT & ~1) : 1 + t * (kSlots / WT);
+  }
+  static constexpr int load_slot(int j) { return j < 6 ? kSyncAt + 2 + 4 * j : kSlots - 4 + 2 * (j - 6); }
+  static_assert(WV == 8 && WT == 4 && NQ == 8, "the slot tables above are laid out for 8 x 4 blocks and 8 loads");
+
+  template <bool READ, bool LOAD, bool SYNC>
+  static __device__ __forceinline__ void step(f32x4 (&acc)[WV][WT], vec8 (&a)[WV], const vec8 (&bc)[WT], vec8 (&bn)[WT],
+                                              const unsigned char* rd_c, const unsigned char* rd_e, const Source& src,
+                                              int koff, unsigned lds_base, int ld_stage, int wave) {
+    static_for<WV * WT>([&](auto idx_c) {
+      constexpr int idx = decltype(idx_c)::value;
+      constexpr int vi = idx / WT, ti = idx % WT;
+      if (SYNC && idx == kSyncAt) {
+        wait_vmcnt<0>();
+        __syncthreads();
+      }
+      acc[vi][ti] = Elem<T>::mfma16(a[vi], bc[ti], acc[vi][ti]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (READ) {
+        static_for<WT>([&](auto t_c) {
+          constexpr int t = decltype(t_c)::value;
+          if (idx == b_slot(SYNC, t)) bn[t] = frag(rd_e + t * 16 * kDmaRowBytes);
+        });
+        static_for<WV>([&](auto v_c) {
+          constexpr int v = decltype(v_c)::value;
+          if (idx == a_slot(SYNC, v)) a[v] = frag(rd_c + v * 16 * kDmaRowBytes);
+        });
+      }
+      if (LOAD) {
+        static_for<NQ>([&](auto j_c) {
+          constexpr int j = decltype(j_c)::value;
+          if (idx == load_slot(j)) issue_one(src, j, koff, lds_base, ld_stage, wave);
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+
+  // Start the ring for the first tile of a span: its first two stages, into ring stages 0 and 1.
+  static __device__ __forceinline__ void prefetch(const Source& src, unsigned char* lds) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) issue_one(src, q, 0, lds_base, 0, wave);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) issue_one(src, q, kDmaBK, lds_base, STAGE_BYTES, wave);
+  }
+
+  // D must be a multiple of 64 and at least 128.  The first two stages of this tile must be in flight or landed in
+  // ring stages buf, 1 - buf (prefetch(), or the previous run()), and nothing else may have touched the ring.
+  // next_tile() is called once, when the class rows of this tile have been fetched for the last time: it points
+  // `src` at the tile whose first stages the rest of this run fetches (or leaves it: those loads then repeat this
+  // tile's first stages and are never read).
+  template <typename NextTile>
+  static __device__ __forceinline__ void run(f32x4 (&acc)[WV][WT], Source& src, unsigned char* lds, int D, int& buf,
+                                             NextTile&& next_tile) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wv = wave / NWT;
+    const int wt = wave % NWT;
+    const int r16 = lane & 15;
+    // this lane's 16-byte chunk of a ring row: (l / 16) for the first half of a stage, + 4 for the second,
+    // XOR-swizzled with (row >> 1) & 7 like the loads place them
+    const int chunk0 = (((lane >> 4) ^ (r16 >> 1)) << 4);
+    const int chunk1 = chunk0 ^ 64;
+    const unsigned char* c_row = lds + (wv * WV * 16 + r16) * kDmaRowBytes;
+    const unsigned char* e_row = lds + (TILE_V + wt * WT * 16 + r16) * kDmaRowBytes;
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi)
+#pragma unroll
+      for (int ti = 0; ti < WT; ++ti)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[vi][ti][r] = 0.0f;
+
+    const int nk = D / kDmaBK;
+    int cur = buf * STAGE_BYTES;
+    wait_vmcnt<NQ>();  // the first stage has landed, the second may be in flight
+    __syncthreads();
+    vec8 a[WV], b0[WT], b1[WT];
+#pragma unroll
+    for (int ti = 0; ti < WT; ++ti) b0[ti] = frag(e_row + cur + chunk0 + ti * 16 * kDmaRowBytes);
+#pragma unroll
+    for (int vi = 0; vi < WV; ++vi) a[vi] = frag(c_row + cur + chunk0 + vi * 16 * kDmaRowBytes);
+
+#pragma unroll 1
+    for (int s = 0; s < nk - 1; ++s) {
+      const int nxt = STAGE_BYTES - cur;
+      step<true, false, false>(acc, a, b0, b1, c_row + cur + chunk1, e_row + cur + chunk1, src, 0, lds_base, 0, wave);
+      if (s == nk - 2) next_tile();
+      const int koff = (s + 2 < nk) ? (s + 2) * kDmaBK : 0;
+      step<true, true, true>(acc, a, b1, b0, c_row + nxt + chunk0, e_row + nxt + chunk0, src, koff, lds_base, cur, wave);
+      cur = nxt;
+    }
+    // the last stage: its second step reads nothing (the next tile's first fragments would sit in registers
+    // through the epilogue) and fetches the second stage of the next tile
+    step<true, false, false>(acc, a, b0, b1, c_row + cur + chunk1, e_row + cur + chunk1, src, 0, lds_base, 0, wave);
+    step<false, true, true>(acc, a, b1, b0, c_row, e_row, src, kDmaBK, lds_base, cur, wave);
+    buf = 1 - cur / STAGE_BYTES;
   }
 };
 

@@ -26,7 +26,7 @@ struct LseFwdParams {
   float* logit_avg;
   float* tile_max;
   float2* partial;  // [nsplit][b] (max2, sum)
-  int64_t b, v, d;
+  int64_t b, v, d, n_rows;
   int64_t stride_e, stride_cv, stride_cd;
   int nrb, nvt, nsplit, nitems, items_per_xcd;
   int stat_cols;
@@ -287,6 +287,237 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The direct-to-LDS kernel on 16 x 16 x 32 MFMAs (DmaLogitTile16): same items, tile, ring and partials as
+// above; a lane holds, per 16-row block ti of its wave, ONE token row (lane % 16) and the 32 classes
+// 16 vi + 4 (lane / 16) + r of the wave's 128.  The epilogue takes two such blocks (32 rows, one row of
+// statistic cells) at a time: 64 soft-capped logits live.
+// ---------------------------------------------------------------------------------------------
+constexpr int kF16WV = 8, kF16WT = 4;  // 16-row blocks per wave: 128 classes x 64 rows
+static_assert(16 * kF16WV * kFwdNWV == kFwdTile && 16 * kF16WT * kFwdNWT == kFwdTile, "tile is 256 x 256");
+
+// Soft-capped logits (log2 domain) of row block ti of a wave: s2[vi][r], 32 values of one token row per lane.
+// Returns this lane's maximum over them; bm[j] accumulates its maximum in the 32-class group j (the classes of a
+// statistic cell).
+template <bool GENERAL, bool CAP>
+__device__ __forceinline__ float row_block_logits_impl(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+                                                       const float* addend, int kq, float (&s2)[kF16WV][4],
+                                                       float (&bm)[kF16WV / 2]) {
+  float tm = -INFINITY;
+#pragma unroll
+  for (int vi = 0; vi < kF16WV; ++vi) {
+    float gm = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = acc[vi][ti][r];
+      bool dead = false;
+      if (GENERAL) {
+        const float add = addend[vi * 16 + 4 * kq + r];
+        dead = (add == -INFINITY);
+        x = dead ? 0.0f : x + add;
+      }
+      float y;
+      if (CAP) {
+        // cap * log2(e) * tanh(x / cap), tanh(u) = 1 - 2 / (1 + exp(2 u))
+        const float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
+        const float w = __builtin_amdgcn_rcpf(1.0f + t);
+        y = fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
+      } else {
+        y = x * kLog2e;
+      }
+      y = dead ? -INFINITY : y;
+      s2[vi][r] = y;
+      gm = fmaxf(gm, y);
+    }
+    bm[vi / 2] = fmaxf(bm[vi / 2], gm);
+    tm = fmaxf(tm, gm);
+  }
+  return tm;
+}
+
+template <bool GENERAL>
+__device__ __forceinline__ float row_block_logits(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+                                                  const float* addend, int kq, float (&s2)[kF16WV][4],
+                                                  float (&bm)[kF16WV / 2]) {
+  // one uniform branch per row block: each arm is straight-line code over all 32 values
+  if (sc.on) return row_block_logits_impl<GENERAL, true>(sc, acc, ti, addend, kq, s2, bm);
+  return row_block_logits_impl<GENERAL, false>(sc, acc, ti, addend, kq, s2, bm);
+}
+
+template <typename T, bool GENERAL, bool WANT_LA>
+__global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdParams p) {
+  using Fast = DmaLogitTile16<T, kF16WV, kF16WT, kFwdNWV, kFwdNWT>;
+  static_assert(!WANT_LA || GENERAL, "the column average uses the general epilogue");
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_addend = reinterpret_cast<float*>(smem + Fast::LDS_BYTES);  // [2][256]
+
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  if (slot >= p.items_per_xcd) return;
+  const int item = xcd * p.items_per_xcd + slot;
+  if (item >= p.nitems) return;
+  const int rb = item / p.nsplit;
+  const int split = item % p.nsplit;
+  const int vt_begin = static_cast<int>((static_cast<int64_t>(p.nvt) * split) / p.nsplit);
+  const int vt_end = static_cast<int>((static_cast<int64_t>(p.nvt) * (split + 1)) / p.nsplit);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wv = wave / kFwdNWT;
+  const int wt = wave % kFwdNWT;
+  const int r16 = lane & 15;
+  const int kq = lane >> 4;
+  const int64_t t0 = static_cast<int64_t>(rb) * kFwdTile;
+  const int64_t wrow0 = t0 + wt * (16 * kF16WT);  // first row of this wave
+
+  // Per-lane byte offsets of the direct-to-LDS loads (the launcher has checked that they fit 32 bits): token rows
+  // relative to e, class rows relative to the first class of the tile.
+  typename Fast::Source src;
+  src.e_base = reinterpret_cast<const unsigned char*>(p.e);
+  const unsigned chunk_bytes = 2u * static_cast<unsigned>(Fast::chunk_elems(wave, lane));
+#pragma unroll
+  for (int q = Fast::NQC; q < Fast::NQ; ++q) {
+    int64_t i = t0 + Fast::row_of(q, wave, lane);
+    i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
+    const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
+    src.off[q] = static_cast<unsigned>(row * p.stride_e * 2) + chunk_bytes;
+  }
+  auto set_class_tile = [&](int64_t v0) {
+    src.c_base = reinterpret_cast<const unsigned char*>(p.c) + v0 * p.stride_cv * 2;
+    const int left = static_cast<int>(min(p.v - v0, static_cast<int64_t>(kFwdTile)));  // classes of this tile inside V
+#pragma unroll
+    for (int q = 0; q < Fast::NQC; ++q) {
+      // classes past the end repeat the last one; masked in the epilogue
+      const int vr = min(Fast::row_of(q, wave, lane), left - 1);
+      src.off[q] = static_cast<unsigned>(vr) * static_cast<unsigned>(p.stride_cv * 2) + chunk_bytes;
+    }
+  };
+
+  float m2[kF16WT], sum[kF16WT];
+#pragma unroll
+  for (int ti = 0; ti < kF16WT; ++ti) {
+    m2[ti] = -INFINITY;
+    sum[ti] = 0.0f;
+  }
+
+  int buf = 0;
+  set_class_tile(static_cast<int64_t>(vt_begin) * kFwdTile);
+  Fast::prefetch(src, smem);
+
+  for (int vt = vt_begin; vt < vt_end; ++vt) {
+    const int64_t v0 = static_cast<int64_t>(vt) * kFwdTile;
+    float* addend = s_addend + (vt & 1) * kFwdTile;
+    if (GENERAL) {
+      // Written before the main loop, whose barriers publish it; the other buffer may still be read
+      // by a wave that is finishing the previous tile.
+      if (tid < kFwdTile) {
+        const int64_t vg = v0 + tid;
+        float a = -INFINITY;
+        if (vg < p.v) a = (p.bias != nullptr) ? Elem<T>::to_float(p.bias[vg]) : 0.0f;
+        addend[tid] = a;
+      }
+    }
+    f32x4 acc[kF16WV][kF16WT];
+    Fast::run(acc, src, smem, static_cast<int>(p.d), buf, [&] {
+      if (vt + 1 < vt_end) set_class_tile(v0 + kFwdTile);
+    });
+
+    // ---- epilogue: (bias, mask,) soft-cap, online max / sum-exp ---------------------------------
+    const int64_t vw0 = v0 + wv * (16 * kF16WV);  // first class of this wave
+    const float* wave_addend = addend + wv * (16 * kF16WV);
+#pragma unroll
+    for (int tp = 0; tp < kF16WT / 2; ++tp) {
+      float bm[kF16WV / 2];  // this lane's maxima in the four statistic cells of this row pair
+#pragma unroll
+      for (int j = 0; j < kF16WV / 2; ++j) bm[j] = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int ti = 2 * tp + u;
+        __builtin_amdgcn_sched_barrier(0);  // keep each row block's register use to itself
+        float s2[kF16WV][4];
+        const float tm = row_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, kq, s2, bm);
+        if (WANT_LA) {
+          // Column sums over the 16 rows of this block, in natural-log units, added to the running average right away.
+          const float ok = (wrow0 + ti * 16 + r16 < p.b) ? 1.0f : 0.0f;
+          const float inv_b = kLn2 / static_cast<float>(p.b);
+          float* avg = p.logit_avg + vw0 + 4 * kq;  // this lane group's first class of the wave
+          const int left = static_cast<int>(min(p.v - vw0, static_cast<int64_t>(16 * kF16WV))) - 4 * kq;
+#pragma unroll
+          for (int vi = 0; vi < kF16WV; ++vi) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int cls = vi * 16 + r;
+              float cs = (s2[vi][r] == -INFINITY) ? 0.0f : s2[vi][r] * ok;
+#pragma unroll
+              for (int off = 8; off >= 1; off >>= 1) cs += __shfl_xor(cs, off, 64);
+              if (r16 == 0 && cls < left) unsafeAtomicAdd(avg + cls, cs * inv_b);
+            }
+          }
+        }
+        const float mn = fmaxf(m2[ti], tm);
+        const float ms = (mn == -INFINITY) ? 0.0f : mn;
+        float part = 0.0f;
+#pragma unroll
+        for (int vi = 0; vi < kF16WV; ++vi)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(s2[vi][r] - ms);
+        sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + part;
+        m2[ti] = mn;
+      }
+
+      if (p.tile_max != nullptr) {
+        // max over the 32 rows x 32 classes of each statistic cell of this (wave, row pair)
+        const int64_t prow = wrow0 + tp * 32;
+        float cell[kF16WV / 2];
+#pragma unroll
+        for (int j = 0; j < kF16WV / 2; ++j) cell[j] = wave_max(bm[j]);
+        if (lane < kF16WV / 2 && prow < p.b && vw0 + lane * 32 < p.v) {
+          float mine = cell[0];
+#pragma unroll
+          for (int j = 1; j < kF16WV / 2; ++j) mine = (lane == j) ? cell[j] : mine;
+          p.tile_max[(prow / CCE_STAT_ROWS) * p.stat_cols + vw0 / CCE_STAT_COLS + lane] = mine * kLn2;
+        }
+      }
+    }
+  }
+
+  // the loads issued under the last tile (its own first stages once more) must land before the ring is reused
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // ---- merge the four lane groups, then the two wave rows, and emit one partial per row -------
+  float2* stage = reinterpret_cast<float2*>(smem);  // [NWT][WT][16]
+#pragma unroll
+  for (int ti = 0; ti < kF16WT; ++ti) {
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+      const float om = __shfl_xor(m2[ti], off, 64);
+      const float os = __shfl_xor(sum[ti], off, 64);
+      const float mn = fmaxf(m2[ti], om);
+      const float ms = (mn == -INFINITY) ? 0.0f : mn;
+      sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + os * __builtin_amdgcn_exp2f(om - ms);
+      m2[ti] = mn;
+    }
+  }
+  if (wv == 1 && kq == 0) {
+#pragma unroll
+    for (int ti = 0; ti < kF16WT; ++ti) stage[(wt * kF16WT + ti) * 16 + r16] = make_float2(m2[ti], sum[ti]);
+  }
+  __syncthreads();
+  if (wv == 0 && kq == 0) {
+#pragma unroll
+    for (int ti = 0; ti < kF16WT; ++ti) {
+      const float2 o = stage[(wt * kF16WT + ti) * 16 + r16];
+      const float mn = fmaxf(m2[ti], o.x);
+      const float ms = (mn == -INFINITY) ? 0.0f : mn;
+      const float s = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + o.y * __builtin_amdgcn_exp2f(o.x - ms);
+      const int64_t i = wrow0 + ti * 16 + r16;
+      if (i < p.b) p.partial[static_cast<int64_t>(split) * p.b + i] = make_float2(mn, s);
+    }
+  }
+}
+
 // lse[i] = ln(2) * (M + log2(sum_s sum_s * 2^(m_s - M))),  M = max_s m_s
 __global__ void lse_merge_kernel(const float2* partial, float* lse, int64_t b, int nsplit) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -314,7 +545,11 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
   const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
+  // the 16 x 16 x 32 kernel addresses token rows by 32-bit byte offsets from e and class rows by offsets from the
+  // first class of a tile; shapes beyond that, and a D of one stage, take the 32 x 32 x 16 kernel
   const bool fast = aligned && (p.d % kDmaBK == 0);
+  const bool fast16 = fast && (p.d >= 2 * kDmaBK) && (p.n_rows * p.stride_e * 2 < (int64_t(1) << 32)) &&
+                      (256 * p.stride_cv * 2 < (int64_t(1) << 32));
   const bool general = want_la || (p.bias != nullptr) || (p.v % Tile::TILE_V != 0);
   const int grid = p.items_per_xcd * 8;
   hipError_t err;
@@ -326,7 +561,19 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
     if (err != hipSuccess) return status_from_hip(err);                                           \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                           \
   } while (0)
-  if (fast) {
+#define CCE_LAUNCH_FWD16(GE, LA)                                                                  \
+  do {                                                                                            \
+    auto kern = lse_forward16_kernel<T, GE, LA>;                                                  \
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+    if (err != hipSuccess) return status_from_hip(err);                                           \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                      \
+  } while (0)
+  if (fast16) {
+    if (want_la) CCE_LAUNCH_FWD16(true, true);
+    else if (general) CCE_LAUNCH_FWD16(true, false);
+    else CCE_LAUNCH_FWD16(false, false);
+  } else if (fast) {
     if (want_la) CCE_LAUNCH_FWD(true, true, true, true);
     else if (general) CCE_LAUNCH_FWD(true, true, true, false);
     else CCE_LAUNCH_FWD(true, true, false, false);
@@ -336,6 +583,7 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
     if (want_la) CCE_LAUNCH_FWD(false, false, true, true); else CCE_LAUNCH_FWD(false, false, true, false);
   }
 #undef CCE_LAUNCH_FWD
+#undef CCE_LAUNCH_FWD16
   return status_from_hip(hipGetLastError());
 }
 
@@ -378,6 +626,7 @@ static int lse_forward_impl(const void* e, const void* c, const void* bias, cons
   p.b = b;
   p.v = v;
   p.d = d;
+  p.n_rows = n_rows;
   p.stride_e = stride_e;
   p.stride_cv = stride_cv;
   p.stride_cd = stride_cd;
