@@ -534,13 +534,34 @@ struct DmaLogitTile16 {
   static __device__ __forceinline__ int row_of(int q, int wave, int lane) { return Base::row_of(q, wave, lane); }
   static __device__ __forceinline__ int chunk_elems(int wave, int lane) { return Base::chunk_elems(wave, lane); }
 
-  // Where the loads of a tile come from: per load a 32-bit byte offset of this lane's row and chunk, relative to a
-  // wave-uniform base -- the first class row of the tile for the class loads, the matrix of token rows for the others.
+  // Where the loads of a tile come from.  A load fetches 8 rows x 128 bytes; its address is a wave-uniform 64-bit base
+  // (scalar registers) plus a 32-bit byte offset per lane.  Token rows are gathered, so each of their loads has an
+  // offset of its own relative to the matrix (e_off).  Class rows are consecutive: the base of load q is the first
+  // row of its block of 8 and the lane adds (its row in the block) x (row stride) + (its chunk); for a tile that
+  // reaches past the last class the block is moved back inside and the row clamped to c_lim[q], so that every
+  // lane reads a row that exists (what it feeds is masked in the epilogue).  Only c_blk / c_lim change from tile
+  // to tile, on the scalar unit.
   struct Source {
-    unsigned off[NQ];
-    const unsigned char* c_base;
+    unsigned e_off[NQ - NQC];
     const unsigned char* e_base;
+    const unsigned char* c_blk[NQC];
+    int c_lim[NQC];
+    unsigned c_stride_bytes;
+    unsigned row_in_block;  // lane >> 3
+    unsigned chunk_bytes;   // byte offset of this lane's 16-byte chunk inside a 128-byte row segment
   };
+
+  // Points the class loads of `src` at the tile whose first class row is `tile` and which has `left` >= 1 classes
+  // inside the matrix (256 or more: a whole tile).
+  static __device__ __forceinline__ void set_class_tile(Source& src, const unsigned char* tile, int left, int wave) {
+#pragma unroll
+    for (int q = 0; q < NQC; ++q) {
+      const int first = 8 * (q * NW + wave);
+      const int blk = min(first, left - 1);
+      src.c_blk[q] = tile + static_cast<int64_t>(blk) * src.c_stride_bytes;
+      src.c_lim[q] = left - 1 - blk;
+    }
+  }
 
   static __device__ __forceinline__ vec8 frag(const unsigned char* p) {
     return __builtin_bit_cast(vec8, *reinterpret_cast<const uint4*>(p));
@@ -549,9 +570,14 @@ struct DmaLogitTile16 {
   // Load q of one stage, columns [k0, k0 + 64), into ring stage `stage_off`.
   static __device__ __forceinline__ void issue_one(const Source& src, int q, int k0, unsigned lds_base, int stage_off,
                                                    int wave) {
-    const int blk = (q < NQC) ? (q * NW + wave) : (TILE_V / 8 + (q - NQC) * NW + wave);
-    const unsigned char* base = ((q < NQC) ? src.c_base : src.e_base) + 2 * k0;
-    lds_dma16_sbase(base, src.off[q], lds_base + stage_off + blk * 1024);
+    if (q < NQC) {
+      const unsigned row = min(src.row_in_block, static_cast<unsigned>(src.c_lim[q]));
+      lds_dma16_sbase(src.c_blk[q] + 2 * k0, row * src.c_stride_bytes + src.chunk_bytes,
+                      lds_base + stage_off + (q * NW + wave) * 1024);
+    } else {
+      lds_dma16_sbase(src.e_base + 2 * k0, src.e_off[q - NQC],
+                      lds_base + stage_off + (TILE_V / 8 + (q - NQC) * NW + wave) * 1024);
+    }
   }
 
   // One step: WV x WT MFMAs on the class fragments a[] and the token fragments bc[]; under them, at most one

@@ -350,6 +350,10 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
   static_assert(!WANT_LA || GENERAL, "the column average uses the general epilogue");
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_addend = reinterpret_cast<float*>(smem + Fast::LDS_BYTES);  // [2][256]
+  // The running (max, sum-exp) of this lane's kF16WT token rows lives in LDS between the epilogues: [ti][thread].
+  // Eight registers fewer across the main loop, which is what lets the loop and the epilogue go without spills
+  // (a reload from scratch memory makes the compiler wait for ALL loads in flight, the ring's included).
+  float2* s_run = reinterpret_cast<float2*>(smem + Fast::LDS_BYTES + kFwdBiasBytes) + threadIdx.x;
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -363,7 +367,9 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  // wave-uniform, and known to the compiler as such: everything derived from it (row and class offsets of the
+  // wave, addresses of the statistic cells) then lives in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wv = wave / kFwdNWT;
   const int wt = wave % kFwdNWT;
   const int r16 = lane & 15;
@@ -371,35 +377,26 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
   const int64_t t0 = static_cast<int64_t>(rb) * kFwdTile;
   const int64_t wrow0 = t0 + wt * (16 * kF16WT);  // first row of this wave
 
-  // Per-lane byte offsets of the direct-to-LDS loads (the launcher has checked that they fit 32 bits): token rows
-  // relative to e, class rows relative to the first class of the tile.
+  // Sources of the direct-to-LDS loads (the launcher has checked that the byte offsets fit 32 bits)
   typename Fast::Source src;
   src.e_base = reinterpret_cast<const unsigned char*>(p.e);
-  const unsigned chunk_bytes = 2u * static_cast<unsigned>(Fast::chunk_elems(wave, lane));
+  src.chunk_bytes = 2u * static_cast<unsigned>(Fast::chunk_elems(wave, lane));
+  src.row_in_block = static_cast<unsigned>(lane >> 3);
+  src.c_stride_bytes = static_cast<unsigned>(p.stride_cv * 2);
 #pragma unroll
   for (int q = Fast::NQC; q < Fast::NQ; ++q) {
     int64_t i = t0 + Fast::row_of(q, wave, lane);
     i = (i < p.b) ? i : p.b - 1;  // rows past the end repeat the last one; their results are dropped
     const int64_t row = p.valids ? static_cast<int64_t>(p.valids[i]) : i;
-    src.off[q] = static_cast<unsigned>(row * p.stride_e * 2) + chunk_bytes;
+    src.e_off[q - Fast::NQC] = static_cast<unsigned>(row * p.stride_e * 2) + src.chunk_bytes;
   }
   auto set_class_tile = [&](int64_t v0) {
-    src.c_base = reinterpret_cast<const unsigned char*>(p.c) + v0 * p.stride_cv * 2;
     const int left = static_cast<int>(min(p.v - v0, static_cast<int64_t>(kFwdTile)));  // classes of this tile inside V
-#pragma unroll
-    for (int q = 0; q < Fast::NQC; ++q) {
-      // classes past the end repeat the last one; masked in the epilogue
-      const int vr = min(Fast::row_of(q, wave, lane), left - 1);
-      src.off[q] = static_cast<unsigned>(vr) * static_cast<unsigned>(p.stride_cv * 2) + chunk_bytes;
-    }
+    Fast::set_class_tile(src, reinterpret_cast<const unsigned char*>(p.c) + v0 * p.stride_cv * 2, left, wave);
   };
 
-  float m2[kF16WT], sum[kF16WT];
 #pragma unroll
-  for (int ti = 0; ti < kF16WT; ++ti) {
-    m2[ti] = -INFINITY;
-    sum[ti] = 0.0f;
-  }
+  for (int ti = 0; ti < kF16WT; ++ti) s_run[ti * kFwdThreads] = make_float2(-INFINITY, 0.0f);
 
   int buf = 0;
   set_class_tile(static_cast<int64_t>(vt_begin) * kFwdTile);
@@ -455,20 +452,23 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
             }
           }
         }
-        const float mn = fmaxf(m2[ti], tm);
+        const float2 run = s_run[ti * kFwdThreads];
+        const float mn = fmaxf(run.x, tm);
         const float ms = (mn == -INFINITY) ? 0.0f : mn;
         float part = 0.0f;
 #pragma unroll
         for (int vi = 0; vi < kF16WV; ++vi)
 #pragma unroll
           for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(s2[vi][r] - ms);
-        sum[ti] = sum[ti] * __builtin_amdgcn_exp2f(m2[ti] - ms) + part;
-        m2[ti] = mn;
+        s_run[ti * kFwdThreads] = make_float2(mn, run.y * __builtin_amdgcn_exp2f(run.x - ms) + part);
       }
 
       if (p.tile_max != nullptr) {
         // max over the 32 rows x 32 classes of each statistic cell of this (wave, row pair)
-        const int64_t prow = wrow0 + tp * 32;
+        int64_t prow = wrow0 + tp * 32;
+        // (the compiler would otherwise form the per-lane address of every cell row before the tile loop and
+        // hold the pairs of registers through the main loop)
+        asm volatile("" : "+s"(prow));
         float cell[kF16WV / 2];
 #pragma unroll
         for (int j = 0; j < kF16WV / 2; ++j) cell[j] = wave_max(bm[j]);
@@ -488,6 +488,13 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
 
   // ---- merge the four lane groups, then the two wave rows, and emit one partial per row -------
   float2* stage = reinterpret_cast<float2*>(smem);  // [NWT][WT][16]
+  float m2[kF16WT], sum[kF16WT];
+#pragma unroll
+  for (int ti = 0; ti < kF16WT; ++ti) {
+    const float2 run = s_run[ti * kFwdThreads];
+    m2[ti] = run.x;
+    sum[ti] = run.y;
+  }
 #pragma unroll
   for (int ti = 0; ti < kF16WT; ++ti) {
 #pragma unroll
@@ -545,6 +552,7 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
   const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
+  const int lds16 = lds + kF16WT * kFwdThreads * static_cast<int>(sizeof(float2));  // + the running (max, sum) pairs
   // the 16 x 16 x 32 kernel addresses token rows by 32-bit byte offsets from e and class rows by offsets from the
   // first class of a tile; shapes beyond that, and a D of one stage, take the 32 x 32 x 16 kernel
   const bool fast = aligned && (p.d % kDmaBK == 0);
@@ -565,9 +573,9 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   do {                                                                                            \
     auto kern = lse_forward16_kernel<T, GE, LA>;                                                  \
     err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds16);                 \
     if (err != hipSuccess) return status_from_hip(err);                                           \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                      \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds16, stream, p);                    \
   } while (0)
   if (fast16) {
     if (want_la) CCE_LAUNCH_FWD16(true, true);
