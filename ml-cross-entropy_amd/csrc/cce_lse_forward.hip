@@ -296,14 +296,22 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
 constexpr int kF16WV = 8, kF16WT = 4;  // 16-row blocks per wave: 128 classes x 64 rows
 static_assert(16 * kF16WV * kFwdNWV == kFwdTile && 16 * kF16WT * kFwdNWT == kFwdTile, "tile is 256 x 256");
 
-// Soft-capped logits (log2 domain) of row block ti of a wave: s2[vi][r], 32 values of one token row per lane.
-// Returns this lane's maximum over them; bm[j] accumulates its maximum in the 32-class group j (the classes of a
-// statistic cell).
-template <bool GENERAL, bool CAP>
-__device__ __forceinline__ float row_block_logits_impl(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
-                                                       const float* addend, int kq, float (&s2)[kF16WV][4],
-                                                       float (&bm)[kF16WV / 2]) {
+// One row block (16 token rows x the wave's 128 classes; 32 values of ONE row per lane) of the epilogue: soft-cap,
+// the lane's maximum per 32-class group (for the statistic cells) and the update of the row's running (max, sum-exp).
+//
+// FIXED: soft-capping with a cap small enough that 2^(-2 cap log2(e)) is a normal float.  Soft-capped logits never
+// exceed the cap, so the cap itself is the reference of every row's sum of exponentials -- no running maximum, no
+// rescaling, and with w = 1 / (1 + exp(2 x / cap)):  softcap(x) - cap = -2 cap w, so a term of the sum is
+// 2^(-2 cap log2(e) w): two instructions fewer per logit than soft-cap, subtract, exponentiate.  The cell maxima are
+// taken on the raw logits (soft-capping is monotone) and soft-capped once per cell.  The running pair then holds
+// (cap log2(e), sum) and merges with the other spans' pairs like any other.
+template <bool GENERAL, bool CAP, bool FIXED, bool WANT_S2>
+__device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+                                               const float* addend, int kq, float2& run, float (&bm)[kF16WV / 2],
+                                               float (&s2)[kF16WV][4]) {
+  float y[kF16WV][4];
   float tm = -INFINITY;
+  float part = 0.0f;
 #pragma unroll
   for (int vi = 0; vi < kF16WV; ++vi) {
     float gm = -INFINITY;
@@ -316,32 +324,55 @@ __device__ __forceinline__ float row_block_logits_impl(const Softcap& sc, const 
         dead = (add == -INFINITY);
         x = dead ? 0.0f : x + add;
       }
-      float y;
-      if (CAP) {
-        // cap * log2(e) * tanh(x / cap), tanh(u) = 1 - 2 / (1 + exp(2 u))
+      if (FIXED) {
         const float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
         const float w = __builtin_amdgcn_rcpf(1.0f + t);
-        y = fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
+        const float term = __builtin_amdgcn_exp2f(w * (-2.0f * sc.out_scale));
+        part += dead ? 0.0f : term;
+        gm = fmaxf(gm, dead ? -INFINITY : x);
+        if (WANT_S2) s2[vi][r] = dead ? -INFINITY : fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
       } else {
-        y = x * kLog2e;
+        float v;
+        if (CAP) {
+          // cap * log2(e) * tanh(x / cap), tanh(u) = 1 - 2 / (1 + exp(2 u))
+          const float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
+          const float w = __builtin_amdgcn_rcpf(1.0f + t);
+          v = fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
+        } else {
+          v = x * kLog2e;
+        }
+        v = dead ? -INFINITY : v;
+        y[vi][r] = v;
+        if (WANT_S2) s2[vi][r] = v;
+        gm = fmaxf(gm, v);
       }
-      y = dead ? -INFINITY : y;
-      s2[vi][r] = y;
-      gm = fmaxf(gm, y);
     }
     bm[vi / 2] = fmaxf(bm[vi / 2], gm);
     tm = fmaxf(tm, gm);
   }
-  return tm;
+  if (FIXED) {
+    run.x = sc.out_scale;
+    run.y += part;
+  } else {
+    const float mn = fmaxf(run.x, tm);
+    const float ms = (mn == -INFINITY) ? 0.0f : mn;
+#pragma unroll
+    for (int vi = 0; vi < kF16WV; ++vi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(y[vi][r] - ms);
+    run.y = run.y * __builtin_amdgcn_exp2f(run.x - ms) + part;
+    run.x = mn;
+  }
 }
 
-template <bool GENERAL>
-__device__ __forceinline__ float row_block_logits(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
-                                                  const float* addend, int kq, float (&s2)[kF16WV][4],
-                                                  float (&bm)[kF16WV / 2]) {
-  // one uniform branch per row block: each arm is straight-line code over all 32 values
-  if (sc.on) return row_block_logits_impl<GENERAL, true>(sc, acc, ti, addend, kq, s2, bm);
-  return row_block_logits_impl<GENERAL, false>(sc, acc, ti, addend, kq, s2, bm);
+// One uniform branch per row block: each arm is straight-line code over all 32 values.
+template <bool GENERAL, bool WANT_S2>
+__device__ __forceinline__ void row_block(const Softcap& sc, bool fixed_ref, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+                                          const float* addend, int kq, float2& run, float (&bm)[kF16WV / 2],
+                                          float (&s2)[kF16WV][4]) {
+  if (fixed_ref) row_block_impl<GENERAL, true, true, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
+  else if (sc.on) row_block_impl<GENERAL, true, false, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
+  else row_block_impl<GENERAL, false, false, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
 }
 
 template <typename T, bool GENERAL, bool WANT_LA>
@@ -395,6 +426,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
     Fast::set_class_tile(src, reinterpret_cast<const unsigned char*>(p.c) + v0 * p.stride_cv * 2, left, wave);
   };
 
+  // 2^(-2 cap log2(e)) must stay a normal float: cap log2(e) < 60, i.e. caps up to 41
+  const bool fixed_ref = p.sc.on && p.sc.out_scale < 60.0f;
 #pragma unroll
   for (int ti = 0; ti < kF16WT; ++ti) s_run[ti * kFwdThreads] = make_float2(-INFINITY, 0.0f);
 
@@ -433,7 +466,9 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
         const int ti = 2 * tp + u;
         __builtin_amdgcn_sched_barrier(0);  // keep each row block's register use to itself
         float s2[kF16WV][4];
-        const float tm = row_block_logits<GENERAL>(p.sc, acc, ti, wave_addend, kq, s2, bm);
+        float2 run = s_run[ti * kFwdThreads];
+        row_block<GENERAL, WANT_LA>(p.sc, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
+        s_run[ti * kFwdThreads] = run;
         if (WANT_LA) {
           // Column sums over the 16 rows of this block, in natural-log units, added to the running average right away.
           const float ok = (wrow0 + ti * 16 + r16 < p.b) ? 1.0f : 0.0f;
@@ -452,15 +487,6 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
             }
           }
         }
-        const float2 run = s_run[ti * kFwdThreads];
-        const float mn = fmaxf(run.x, tm);
-        const float ms = (mn == -INFINITY) ? 0.0f : mn;
-        float part = 0.0f;
-#pragma unroll
-        for (int vi = 0; vi < kF16WV; ++vi)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(s2[vi][r] - ms);
-        s_run[ti * kFwdThreads] = make_float2(mn, run.y * __builtin_amdgcn_exp2f(run.x - ms) + part);
       }
 
       if (p.tile_max != nullptr) {
@@ -476,6 +502,10 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
           float mine = cell[0];
 #pragma unroll
           for (int j = 1; j < kF16WV / 2; ++j) mine = (lane == j) ? cell[j] : mine;
+          if (fixed_ref) {  // the maximum was taken over raw logits
+            const float t = __builtin_amdgcn_exp2f(mine * p.sc.in_scale);
+            mine = fmaf(__builtin_amdgcn_rcpf(1.0f + t), -2.0f * p.sc.out_scale, p.sc.out_scale);
+          }
           p.tile_max[(prow / CCE_STAT_ROWS) * p.stat_cols + vw0 / CCE_STAT_COLS + lane] = mine * kLn2;
         }
       }
