@@ -3,7 +3,10 @@
 One step = forward + backward of ``linear_cross_entropy`` over one batch of synthetic input already
 resident in HBM.  Default workload c2: the Gemma-2-2B-shaped head, E [8192, 2304] bf16 ~ N(0,1),
 C [256000, 2304] bf16 ~ N(0, 0.02), uniform labels, softcap 30, reduction mean, impl="cce" with gradient
-filtering.  ``--workload c1|c3|c4|c5|c5shard`` run the other benchmark configurations.  Prints one JSON line.
+filtering.  ``--workload c1|c3|c4|c5|c5shard`` run the other benchmark configurations; ``--impl`` runs a workload
+under another preset (cce_kahan_full_c, cce_kahan_full_e, cce_kahan, cce_exact), ``--dtype fp16|fp32`` and
+``--bias`` the same inputs in another input type / with a classifier bias, ``--dense-workspace-mb`` caps the
+workspace of the unfiltered backward (memory against time).  Prints one JSON line.
 
 The timing method restates the reference benchmark (benchmark/memory.py:82-112,
 benchmark/__main__.py:41-125): warm-up, then per iteration clear the gradients and run loss + backward.
@@ -22,7 +25,8 @@ for _p in (ROOT, os.path.join(ROOT, "ml-cross-entropy_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk x 2.4 GHz, dense
+PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 4096 flop/clk x 2.4 GHz, dense (bf16 and fp16 alike)
+PEAK_FP32_TFLOPS = 157.3   # dense fp32 matrix peak
 Z_LOSS_WEIGHT = 1e-4
 
 WORKLOADS = {
@@ -101,12 +105,12 @@ def loss_fn(w):
 
     vp = VocabParallelOptions(*w["vp"]) if w["vp"] is not None else None
 
-    def run(e, c, t):
+    def run(e, c, t, bias=None):
         if w["name"] == "c4":
-            nll, lse = linear_cross_entropy(e, c, t, reduction="none", return_lse=True, impl=w["impl"])
+            nll, lse = linear_cross_entropy(e, c, t, bias=bias, reduction="none", return_lse=True, impl=w["impl"])
             return (nll + Z_LOSS_WEIGHT * compute_z_loss(lse, t, reduction="none")).mean()
-        return linear_cross_entropy(e, c, t, softcap=w["softcap"], shift=w["shift"], reduction="mean", impl=w["impl"],
-                                    vocab_parallel_options=vp)
+        return linear_cross_entropy(e, c, t, bias=bias, softcap=w["softcap"], shift=w["shift"], reduction="mean",
+                                    impl=w["impl"], vocab_parallel_options=vp)
 
     return run
 
@@ -176,6 +180,15 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--impl", default=None,
+                    help="run the workload under this preset instead of its own (cce, cce_exact, cce_kahan, "
+                         "cce_kahan_full_c, cce_kahan_full_e, cce_kahan_full_c_full_e)")
+    ap.add_argument("--dtype", default="bf16", choices=("bf16", "fp16", "fp32"),
+                    help="input type of e and c (the bf16 values of the workload, converted)")
+    ap.add_argument("--bias", action="store_true", help="add a classifier bias ~ N(0, 0.02) that wants a gradient")
+    ap.add_argument("--dense-workspace-mb", type=float, default=None,
+                    help="cap the workspace of the unfiltered backward (dz chunk + dE compensation buffer) at this "
+                         "many MB, for presets that ask for it and for a filtered backward that changes to it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--traffic-probe", action="store_true",
@@ -195,13 +208,28 @@ def main():
 
     from cut_cross_entropy import _hip
     from cut_cross_entropy import cce as cce_mod
+    from cut_cross_entropy import cce_backward as bwd_mod
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = make_workload(args.workload)
-    e = w["e"].to(dev).requires_grad_(True)
-    c = w["c"].to(dev).requires_grad_(True)
+    if args.impl is not None:
+        w["impl"] = args.impl
+        w["text"] += f" [run with impl={args.impl}]"
+    if args.dense_workspace_mb is not None:
+        limit = int(args.dense_workspace_mb * 2**20)
+        comp = 2 * w["valid"] * w["D"]  # the 16-bit compensation buffer of dE
+        bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES = limit
+        bwd_mod.DENSE_DZ_BYTES = max(limit - comp, 0)
+        bwd_mod.DENSE_DZ_MIN_CLASSES = 0
+    in_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
+    e = w["e"].to(dev).to(in_dtype).requires_grad_(True)
+    c = w["c"].to(dev).to(in_dtype).requires_grad_(True)
     t = w["t"].to(dev)
+    bias = None
+    if args.bias:
+        gb = torch.Generator().manual_seed(1)
+        bias = (torch.randn((w["V"],), generator=gb) * 0.02).to(torch.bfloat16).to(dev).to(in_dtype).requires_grad_(True)
     B, N, V, D = w["valid"], w["N"], w["V"], w["D"]
     run = loss_fn(w)
     counters = torch.zeros((4,), dtype=torch.int64, device=dev)
@@ -209,7 +237,9 @@ def main():
     def step():
         e.grad = None
         c.grad = None
-        loss = run(e, c, t)
+        if bias is not None:
+            bias.grad = None
+        loss = run(e, c, t, bias)
         loss.backward()
         return loss
 
@@ -239,8 +269,11 @@ def main():
     _hip.set_timers(None)
     ms_per_step = dt / args.steps * 1e3
     cnt = [int(x) for x in counters.tolist()]
-    k_r, k_e, k_c = (cnt[i] / max(cnt[0], 1) for i in (1, 2, 3))
-    kernel_ms = {name: sum(a.elapsed_time(b) for a, b in evs) / len(evs) for name, evs in timers.items()}
+    k_r, k_e, k_c = (min(cnt[i] / max(cnt[0], 1), 1.0) for i in (1, 2, 3))
+    if args.dtype == "fp32":
+        k_r = k_e = k_c = 1.0  # the fp32 path is unfiltered and keeps no counters
+    # per step: a launcher may be called more than once in a step (the fp32 path walks the vocabulary in chunks)
+    kernel_ms = {name: sum(a.elapsed_time(b) for a, b in evs) / args.steps for name, evs in timers.items()}
 
     # ---- loss-path peak memory (allocator peak minus the returned gradients) --------------------
     e.grad = c.grad = None
@@ -249,19 +282,23 @@ def main():
     torch.cuda.reset_peak_memory_stats()
     step()
     torch.cuda.synchronize()
-    peak = torch.cuda.max_memory_allocated() - base
+    peak_bytes = torch.cuda.max_memory_allocated() - base
     grads = e.grad.numel() * e.grad.element_size() + c.grad.numel() * c.grad.element_size()
-    extra_mb = (peak - grads) / 2**20
+    if bias is not None:
+        grads += bias.grad.numel() * bias.grad.element_size()
+    extra_mb = (peak_bytes - grads) / 2**20
 
     traffic, traffic_source = args.traffic, "--traffic" if args.traffic is not None else None
     if traffic is None:
         traffic, traffic_source = measured_traffic(w["name"], _hip.load().cce_source_hash().decode())
 
-    fwd_ms = kernel_ms["lse_forward"]
+    peak = PEAK_FP32_TFLOPS if args.dtype == "fp32" else PEAK_BF16_TFLOPS
+    fwd_ms = kernel_ms["forward_fp32"] if args.dtype == "fp32" else kernel_ms["lse_forward"]
     fwd_flops = 2.0 * B * V * D
     fwd_tflops = fwd_flops / (fwd_ms * 1e-3) / 1e12
-    bwd_name = "backward_dense" if "backward_dense" in kernel_ms else "backward_sparse"
-    bwd_ms = kernel_ms[bwd_name]
+    bwd_parts = [n for n in ("backward_sparse", "backward_dense", "backward_fp32") if n in kernel_ms]
+    bwd_name = "+".join(bwd_parts)
+    bwd_ms = sum(kernel_ms[n] for n in bwd_parts)
     bwd_flops = 2.0 * B * V * D * (k_r + k_e + k_c)
 
     f_alg = 2.0 * B * V * D * (1.0 + k_r + k_e + k_c)
@@ -277,26 +314,32 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {
-            "workload": f"{w['name']}: E[{N},{D}] bf16, C[{V},{D}] bf16 N(0,0.02), {w['text']}, fwd+bwd",
+            "workload": f"{w['name']}: E[{N},{D}] {args.dtype}, C[{V},{D}] {args.dtype} N(0,0.02), {w['text']}"
+                        f"{', classifier bias' if args.bias else ''}, fwd+bwd",
             "valid_tokens": B,
+            "impl": w["impl"],
+            "dense_workspace_limit_mb": None if bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES is None
+            else bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES / 2**20,
         },
         "loss": float(loss),
         "loss_path_peak_mb": extra_mb,
         "kept_tiles": {"k_recompute": k_r, "k_dE": k_e, "k_dC": k_c, "tiles": cnt[0] // max(args.steps, 1)},
         "fwd_bwd_tflops_alg": f_alg / (ms_per_step * 1e-3) / 1e12,
-        "fwd_bwd_frac_alg": f_alg / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-        "fwd_bwd_frac_dense_equiv": f_dense / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "fwd_bwd_frac_alg": f_alg / (ms_per_step * 1e-3) / 1e12 / peak,
+        "fwd_bwd_frac_dense_equiv": f_dense / (ms_per_step * 1e-3) / 1e12 / peak,
         "roofline": {
-            "kernel": "lse_forward_kernel (fused E.C^T + softcap + online log-sum-exp), device events around its "
-                      "launches inside the timed steps",
+            "kernel": ("the fp32 forward (three-way bf16 split of e and c, lse_forward_kernel per vocabulary chunk, merge)"
+                       if args.dtype == "fp32" else
+                       "lse_forward_kernel (fused E.C^T + softcap + online log-sum-exp)")
+                      + ", device events around its launches inside the timed steps",
             "bound": "mfma",
             "achieved": fwd_tflops,
-            "peak": PEAK_BF16_TFLOPS,
+            "peak": peak,
             "unit": "TFLOP/s",
-            "frac": fwd_tflops / PEAK_BF16_TFLOPS,
+            "frac": fwd_tflops / peak,
             "ms_per_launch": fwd_ms,
             "traffic": traffic,
             "traffic_source": traffic_source,
@@ -305,7 +348,8 @@ def main():
             "path": bwd_name,
             "ms": bwd_ms,
             "tflops_alg": bwd_flops / (bwd_ms * 1e-3) / 1e12,
-            "frac_alg": bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "frac_alg": bwd_flops / (bwd_ms * 1e-3) / 1e12 / peak,
+            "parts_ms": {n: kernel_ms[n] for n in bwd_parts},
         },
     }
     if not args.no_cpu_baseline:

@@ -98,13 +98,24 @@ int cce_lse_forward(const void* e, const void* c, const void* bias, const int32_
  * return CCE_ERR_STATIC_SCRATCH_LIMIT (c2 needs 0.5 MB, E [65536, 3584] x C [152064, 3584] 2 MB).
  * All calls on one GPU share the array: calls that overlap in time on one GPU race; calls on one
  * stream, or otherwise ordered, are safe (a launch writes every partial before reading it, so nothing
- * carries over from the previous call).
+ * carries over from the previous call).  With logit_avg the call also launches a small fill kernel for it and the
+ * forward adds to it with float atomics, as cce_lse_forward does.
  */
 int cce_lse_forward_static(const void* e, const void* c, const void* bias, const int32_t* valids,
                            float* lse, float* logit_avg, float* tile_max,
                            int64_t n_rows, int64_t b, int64_t v, int64_t d,
                            int64_t stride_e, int64_t stride_cv, int64_t stride_cd,
                            float softcap, int dtype, void* stream);
+
+/*
+ * Set-up of cce_lse_forward_static for the CURRENT device: looks up the address of that device's copy of the
+ * static array (hipGetSymbolAddress, which may load the code object) and keeps it.  cce_lse_forward_static does
+ * the same by itself on its first call on a device; a caller whose first call would fall inside a HIP graph
+ * capture, where nothing may be loaded, calls this once per device beforehand.  Both look the array up for the
+ * device that is current in the calling thread: the caller makes the device of `stream` current first.
+ * No counterpart in the reference (see cce_lse_forward_static).
+ */
+int cce_lse_forward_static_init(void);
 
 /*
  * out[i] = softcap(-(e[valids[i]] . c[t_i]) - bias[t_i]),  t_i = targets[valids[i] + shift] - target_offset;

@@ -1407,8 +1407,8 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
 #define CCE_LAUNCH(KERN, LDS, GRID)                                                                 \
   do {                                                                                              \
     auto kern = KERN;                                                                               \
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                  \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, LDS);                     \
+    static LdsLimitOnce lds_limit;                                                            \
+    err = lds_limit.set(kern, LDS);                                        \
     if (err != hipSuccess) return status_from_hip(err);                                             \
     hipLaunchKernelGGL(kern, dim3(GRID), dim3(kBwdThreads), LDS, stream, p);                        \
   } while (0)
@@ -1445,12 +1445,14 @@ extern "C" int cce_backward(const void* e, const void* c, const void* bias,
       const unsigned grid = static_cast<unsigned>(q.nvg);
       if (dtype == CCE_DTYPE_BF16) {
         auto kern = bwd_owner_fast_kernel<BF16, false, true>;
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kFLightLdsBytes);
+        static LdsLimitOnce lds_limit;
+        err = lds_limit.set(kern, kFLightLdsBytes);
         if (err != hipSuccess) return status_from_hip(err);
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kBwdThreads), kFLightLdsBytes, stream, q);
       } else {
         auto kern = bwd_owner_fast_kernel<F16, false, true>;
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kFLightLdsBytes);
+        static LdsLimitOnce lds_limit;
+        err = lds_limit.set(kern, kFLightLdsBytes);
         if (err != hipSuccess) return status_from_hip(err);
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kBwdThreads), kFLightLdsBytes, stream, q);
       }

@@ -9,6 +9,7 @@
 // statistics a register-local reduction.
 #pragma once
 
+#include <atomic>
 #include <utility>
 
 #include <hip/hip_runtime.h>
@@ -701,6 +702,39 @@ struct DmaLogitTile16 {
   }
 };
 
+inline int status_from_hip(hipError_t e) { return e == hipSuccess ? CCE_OK : static_cast<int>(e); }
+
+// The dynamic LDS limit of a kernel (hipFuncAttributeMaxDynamicSharedMemorySize), set once per kernel and device
+// instead of with every launch: it is a driver call, and the unfiltered backward launches dozens of kernels per
+// step.  One object per kernel, a static at its launch site.
+struct LdsLimitOnce {
+  std::atomic<uint64_t> done{0};  // one bit per device
+  template <typename K>
+  hipError_t set(K kern, int bytes) {
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    const uint64_t bit = uint64_t(1) << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return err;
+  }
+};
+
+// Compute units of the current device (256 on an MI355X), looked up once per device.
+inline int compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  int n = cached[dev & 63].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev & 63].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 // Vocabulary spans per row block for the kernels that cut the (row block, vocabulary) plane into
 // items of one row block x one span of tiles.  Two things are weighed: the rounds of 256 workgroups
 // the items make, and the L2 traffic of the 32 workgroups that run on one XCD at a time, which cover
@@ -708,7 +742,7 @@ struct DmaLogitTile16 {
 // least for s = 4 .. 8.  The weight 0.165 is fitted to measurements at E [65536, 3584] x C [152064, 3584]
 // (1, 2, 4, 8, 16 spans: 70.8, 62.5, 53.9, 56.8, 59.4 ms).
 inline int choose_span_count(int nrb, int nvt) {
-  const int num_cu = 256;
+  const int num_cu = compute_units();  // (the size query and the launch must see the same device)
   int best = 1;
   double best_cost = 1e300;
   const int max_split = nvt < 64 ? nvt : 64;
@@ -726,8 +760,6 @@ inline int choose_span_count(int nrb, int nvt) {
   }
   return best;
 }
-
-inline int status_from_hip(hipError_t e) { return e == hipSuccess ? CCE_OK : static_cast<int>(e); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -296,8 +296,8 @@ int dense_dz_launch(const void* e, const void* c, const void* bias,
 #define CCE_LAUNCH_DZ2(TT, GE, O32)                                                               \
   do {                                                                                            \
     auto kern = dense_dz_kernel<TT, GE, O32>;                                                     \
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+    static LdsLimitOnce lds_limit;                                                            \
+    err = lds_limit.set(kern, lds);                                        \
     if (err != hipSuccess) return status_from_hip(err);                                           \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kDzThreads), lds, stream, p);                       \
   } while (0)

@@ -594,16 +594,16 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
 #define CCE_LAUNCH_FWD(FA, AL, GE, LA)                                                            \
   do {                                                                                            \
     auto kern = lse_forward_kernel<T, FA, AL, GE, LA>;                                            \
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);                   \
+    static LdsLimitOnce lds_limit;                                                            \
+    err = lds_limit.set(kern, lds);                                        \
     if (err != hipSuccess) return status_from_hip(err);                                           \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, stream, p);                           \
   } while (0)
 #define CCE_LAUNCH_FWD16(GE, LA)                                                                  \
   do {                                                                                            \
     auto kern = lse_forward16_kernel<T, GE, LA>;                                                  \
-    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds16);                 \
+    static LdsLimitOnce lds_limit;                                                            \
+    err = lds_limit.set(kern, lds16);                                        \
     if (err != hipSuccess) return status_from_hip(err);                                           \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds16, stream, p);                    \
   } while (0)
@@ -750,6 +750,11 @@ static int static_scratch_for_current_device(void** out) {
   }
   *out = ptr;
   return CCE_OK;
+}
+
+extern "C" int cce_lse_forward_static_init(void) {
+  void* ws = nullptr;
+  return static_scratch_for_current_device(&ws);
 }
 
 extern "C" int cce_lse_forward_static(const void* e, const void* c, const void* bias, const int32_t* valids,

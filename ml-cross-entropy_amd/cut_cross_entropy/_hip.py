@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
 STAT_ROWS = 32
 STAT_COLS = 32
@@ -42,6 +42,7 @@ _SIGNATURES = {
         [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
         + [_i64] * 4 + [_i64] * 3 + [_f32, _i32, _ptr],
     ),
+    "cce_lse_forward_static_init": (_i32, []),
     "cce_indexed_neg_dot": (
         _i32,
         [_ptr] * 6 + [_i64] * 4 + [_i64] * 3 + [_i64, _i64, _f32, _i32, _ptr],

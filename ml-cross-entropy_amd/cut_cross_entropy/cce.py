@@ -118,7 +118,8 @@ class LinearCrossEntropyFunction(torch.autograd.Function):
             assert c.dtype == torch.float32, "e and c must have the same dtype"
             _hip.require_gpu_tensor("e", e)
             e = e.contiguous()
-            lse = fp32_path.fp32_lse(e, c, bias, params.valids, params.softcap)
+            with _hip.timed("forward_fp32", e.device):
+                lse = fp32_path.fp32_lse(e, c, bias, params.valids, params.softcap)
             neg_dot = fp32_path.fp32_indexed_neg_dot(e, c, bias, params.targets, params.valids, params.shift,
                                                      params.softcap, params.first_class)
         else:
@@ -147,9 +148,11 @@ class LinearCrossEntropyFunction(torch.autograd.Function):
             d_lse = d_lse.reshape(-1)
 
         if ctx.is_fp32:
-            de, dc, dbias = fp32_path.fp32_backward(
-                e, c, bias, lse, d_loss, d_lse, valids, targets, params.shift, params.first_class, params.softcap,
-                scale, e_info.requires_grad, c_info.requires_grad, bias_info is not None and bias_info.requires_grad)
+            with _hip.timed("backward_fp32", e.device):
+                de, dc, dbias = fp32_path.fp32_backward(
+                    e, c, bias, lse, d_loss, d_lse, valids, targets, params.shift, params.first_class,
+                    params.softcap, scale, e_info.requires_grad, c_info.requires_grad,
+                    bias_info is not None and bias_info.requires_grad)
             if dbias is not None:
                 dbias = dbias.to(bias_info.dtype)
         else:

@@ -34,26 +34,33 @@ def _dz_budget(B: int) -> int:
 # the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
 # statistic can hold a probability above filter_eps for E [8192, 2304] x C [256000, 2304], and at 0.083 for
 # E [16384, 4096] x C [128256, 4096], where a workgroup of the ownership kernels covers D in two slices and
-# recomputes its logits for each.  Above DENSE_WHEN_FLAGGED_ABOVE / slices the backward runs unfiltered; an
+# recomputes its logits for each.  Above DENSE_WHEN_FLAGGED_ABOVE / slices a FILTERED backward runs unfiltered; an
 # unfiltered gradient is the exact one, so nothing is lost.  None switches the test off.
 #
-# The fraction is measured on the device (cce_count_flagged_cells over the forward's statistic) and read on the
-# host WITHOUT waiting for the device: every filtered backward enqueues the count and an asynchronous copy of
-# it to pinned host memory, and uses the most recent count that has arrived -- normally that of the step
-# before.  The soft-max distribution of a model moves slowly, so a decision that lags one step is as good;
-# the first backward of a shape has no count yet and takes the ownership kernels (always correct, slower when
-# the soft-max is flat).  FILTERED_BACKWARD_PATH pins the choice: "sparse" or "dense" instead of "auto".
+# The fraction is measured on the device (cce_count_flagged_cells over the forward's statistic) and the choice is
+# a function of the data alone, the same on every run: every filtered backward enqueues the count of ITS cells and
+# an asynchronous copy of it to pinned host memory; the FIRST backward of a (device, V, D, dtype) waits for its own
+# count (once per shape and process, as the reference's first call waits for its autotuner), every later one uses
+# the count of the backward before it, which has long arrived (a soft-max distribution moves slowly, so a decision
+# that lags one step is as good).  Identical inputs therefore take the same path, and give the same bits, on the
+# first call and on the tenth.  While a HIP graph is being captured nothing is measured or read: the capture
+# takes the path of the last backward of that shape outside a capture (the ownership kernels if there was none),
+# and the graph replays that path.  FILTERED_BACKWARD_PATH pins the choice: "sparse" or "dense" instead of "auto".
 DENSE_WHEN_FLAGGED_ABOVE = 0.17
 FILTERED_BACKWARD_PATH = "auto"
-# The unfiltered path's workspace (dz chunk + compensation buffer) grows with the number of rows; where memory
-# matters more than time, a byte count here keeps a FILTERED backward whose workspace would be larger on the
-# ownership kernels (which need one bit per 32 x 32 sub-tile and nothing else).  None: no limit.
-DENSE_WORKSPACE_LIMIT_BYTES: Optional[int] = None
+# A filtered backward that changes to the unfiltered path BY ITSELF may take at most this much workspace (the dz
+# chunk, plus the [B, D] 16-bit compensation buffer of dE): the ownership kernels need well under 16 MB, and a
+# caller who picked a filtered preset did not ask for more.  The dz chunk shrinks to fit (more, smaller chunks:
+# slower); if not even the smallest plan fits -- the compensation buffer alone can exceed it when rows are many --
+# the backward stays on the ownership kernels.  None: no limit.  The presets that ask for unfiltered gradients
+# (cce_exact, cce_kahan_full_*) are not bound by it: their dz chunk is DENSE_DZ_BYTES (the reference's own
+# unfiltered presets take fp32 copies of dE and dC, 2.3 GB at E [8192, 2304] x C [256000, 2304]).
+DENSE_WORKSPACE_LIMIT_BYTES: Optional[int] = 256 << 20
 _OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
 
 class _FlaggedMonitor:
-    """Latest measured fraction of flagged cells for one (device, V, D, dtype), read without a host wait."""
+    """Fraction of flagged cells of the latest backward of one (device, V, D, dtype), and the path it chose."""
 
     def __init__(self, device: torch.device):
         self.counter = torch.zeros((1,), dtype=torch.int64, device=device)
@@ -61,16 +68,17 @@ class _FlaggedMonitor:
         self.event = torch.cuda.Event()
         self.pending_cells = 0   # cells of the measurement in flight (0: none)
         self.fraction: Optional[float] = None
+        self.dense: bool = False  # the last choice made outside a capture
 
-    def poll(self) -> Optional[float]:
-        if self.pending_cells and self.event.query():
+    def collect(self) -> None:
+        """Takes in the measurement in flight, waiting for it if it has not arrived."""
+        if self.pending_cells:
+            if not self.event.query():
+                self.event.synchronize()
             self.fraction = int(self.host[0]) / self.pending_cells  # pinned host memory: a plain read
             self.pending_cells = 0
-        return self.fraction
 
     def measure(self, lib, tile_max, lse, B: int, V: int, filter_eps: float, dev: torch.device) -> None:
-        if self.pending_cells or torch.cuda.is_current_stream_capturing():
-            return  # one measurement in flight at a time; none inside a graph capture
         self.counter.zero_()
         with torch.cuda.device(dev):
             status = lib.cce_count_flagged_cells(tile_max.data_ptr(), lse.data_ptr(), B, V, float(filter_eps),
@@ -85,33 +93,54 @@ _monitors: dict = {}
 _monitors_lock = threading.Lock()
 
 
+def reset_backward_path_memory() -> None:
+    """Forgets every measured fraction: the next filtered backward of each shape waits for its own count again."""
+    with _monitors_lock:
+        _monitors.clear()
+
+
+def _auto_dense_dz_budget(lib, B: int, V: int, D: int, de_16bit: bool) -> Optional[int]:
+    """dz chunk bytes a filtered backward may use when it changes to the unfiltered path by itself, or None when
+    even the smallest plan exceeds DENSE_WORKSPACE_LIMIT_BYTES."""
+    budget = _dz_budget(B)
+    if DENSE_WORKSPACE_LIMIT_BYTES is None:
+        return budget
+    comp = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0) - \
+        lib.cce_backward_dense_workspace_bytes(B, V, D, 0, 0)
+    smallest = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0)
+    if smallest > DENSE_WORKSPACE_LIMIT_BYTES:
+        return None
+    return min(budget, DENSE_WORKSPACE_LIMIT_BYTES - comp)
+
+
 def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, filter_eps: float, dtype, dev) -> bool:
-    """The dense / sparse choice of a filtered backward; never waits for the device."""
+    """The dense / sparse choice of a filtered backward."""
     if FILTERED_BACKWARD_PATH != "auto":
         return FILTERED_BACKWARD_PATH == "dense"
     if DENSE_WHEN_FLAGGED_ABOVE is None:
         return False
-    if (DENSE_WORKSPACE_LIMIT_BYTES is not None
-            and lib.cce_backward_dense_workspace_bytes(B, V, D, 1, _dz_budget(B)) > DENSE_WORKSPACE_LIMIT_BYTES):
-        return False
     key = (dev.index, V, D, dtype)
+    capturing = torch.cuda.is_current_stream_capturing()
     with _monitors_lock:
         mon = _monitors.get(key)
+        if capturing:
+            # nothing may be allocated, measured or waited for inside a capture
+            return mon.dense if mon is not None else False
         if mon is None:
-            if torch.cuda.is_current_stream_capturing():
-                return False  # nothing may be allocated for a new shape inside a capture
             mon = _monitors[key] = _FlaggedMonitor(dev)
-        fraction = mon.poll()
-        mon.measure(lib, tile_max, lse, B, V, filter_eps, dev)
-    return fraction is not None and fraction > DENSE_WHEN_FLAGGED_ABOVE / -(-D // _OWNERSHIP_SLICE_COLS)
+        first = mon.fraction is None and not mon.pending_cells
+        if first:
+            mon.measure(lib, tile_max, lse, B, V, filter_eps, dev)  # this backward's own cells ...
+        mon.collect()                                              # ... or those of the backward before
+        fraction = mon.fraction
+        mon.measure(lib, tile_max, lse, B, V, filter_eps, dev)      # for the next backward of this shape
+        mon.dense = fraction is not None and fraction > DENSE_WHEN_FLAGGED_ABOVE / -(-D // _OWNERSHIP_SLICE_COLS)
+        return mon.dense
 
 
-def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_grad, filter_c_grad) -> bool:
-    """The unfiltered backward (cce_backward_dense: dz chunks and the two products as MFMA kernels) runs when
-    nothing that is asked for is filtered and the layout suits the direct-to-LDS kernels."""
-    if filter_eps_or_none(filter_eps) >= 0.0:
-        if (want_de and filter_e_grad) or ((want_dc or want_dbias) and filter_c_grad):
-            return False
+def _dense_layout_ok(e, c) -> bool:
+    """Whether the layout suits the direct-to-LDS kernels of the unfiltered backward (cce_backward_dense: dz chunks
+    and the two products as MFMA kernels)."""
     return (
         e.size(1) % 64 == 0
         and e.stride(0) % 8 == 0
@@ -123,7 +152,7 @@ def _dense_eligible(e, c, want_de, want_dc, want_dbias, filter_eps, filter_e_gra
 
 
 def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
-                    shift, target_offset, softcap):
+                    shift, target_offset, softcap, dz_budget):
     """dE, dC, dBias of the unfiltered backward: one call into the library, which walks the vocabulary in
     chunks (dz of the chunk -> workspace, then the two products as hand-written MFMA kernels; reference:
     cce_backward.py:170-302, there one kernel with atomics).  The workspace -- the dz chunk, plus a 16-bit
@@ -131,7 +160,7 @@ def _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, 
     allocator's peak statistic sees it."""
     V, D = c.size(0), e.size(1)
     de_in_ws = de is not None and de.dtype != torch.float32
-    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_in_ws else 0, _dz_budget(B))
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_in_ws else 0, int(dz_budget))
     workspace = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
     ws_ptr = (workspace.data_ptr() + 255) // 256 * 256
     with torch.cuda.device(dev), _hip.timed("backward_dense", dev):
@@ -218,29 +247,50 @@ def cce_backward_kernel(
         if do.numel() > 1:
             assert dlse.size() == do.size()
 
-    de_dtype = torch.float32 if accum_e_fp32 else e.dtype
-    dc_dtype = torch.float32 if accum_c_fp32 else c.dtype
-    dense = _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad,
-                            bias is not None and bias_info is not None and bias_info.requires_grad,
-                            filter_eps, filter_e_grad, filter_c_grad)
-    if (not dense and tile_max is not None and filter_eps is not None and filter_eps > 0 and lse.numel() > 0
-            and _dense_eligible(e, c, e_info.requires_grad, c_info.requires_grad, False, None, False, False)):
-        n_valid = valids.size(0) if valids is not None else e.size(0)
-        dense = _filtered_backward_runs_dense(lib, tile_max, lse, n_valid, c.size(0), e.size(1), float(filter_eps),
-                                              e.dtype, dev)
-    if dense:
-        # the products of the dense path accumulate in fp32 registers and each output element is written once
-        # (dC, dBias) or summed over the chunks in an fp32 workspace (dE): no fp32 gradient buffers are needed
-        de_dtype, dc_dtype = e_info.dtype, c_info.dtype
     n_valid_rows = valids.size(0) if valids is not None else e.size(0)
+    want_de = e_info.requires_grad
+    want_dc = c_info.requires_grad
+    want_dbias = bias is not None and bias_info is not None and bias_info.requires_grad
+    # dBias follows dC: filtered with it, unfiltered with it
+    filtering = filter_eps_or_none(filter_eps) >= 0.0
+    e_filtered = filtering and filter_e_grad
+    c_filtered = filtering and filter_c_grad
+
+    # Which kernels form which gradient.  An unfiltered gradient is a dense matrix product and goes to
+    # cce_backward_dense; a filtered one goes to the ownership kernels (cce_backward), which pay per surviving
+    # sub-tile.  The reference decides per side inside one kernel (cce_backward.py:211-216, 258-310); here the two
+    # sides of a preset that filters only one of them (cce_kahan_full_c / _full_e) are two library calls.
+    layout_ok = _dense_layout_ok(e, c)
+    de_dense = want_de and layout_ok and not e_filtered
+    dc_dense = (want_dc or want_dbias) and layout_ok and not c_filtered
+    dz_budget = _dz_budget(n_valid_rows)
+    some_filtered = (want_de and not de_dense) or ((want_dc or want_dbias) and not dc_dense)
+    if (some_filtered and layout_ok and tile_max is not None and filter_eps is not None and filter_eps > 0
+            and lse.numel() > 0):
+        # ... unless so many cells are flagged that filtering cannot pay: then everything runs unfiltered (exact)
+        de_16bit = want_de and e_info.dtype != torch.float32
+        auto_budget = dz_budget if (de_dense or dc_dense) else _auto_dense_dz_budget(
+            lib, n_valid_rows, c.size(0), e.size(1), de_16bit)
+        if auto_budget is not None and _filtered_backward_runs_dense(
+                lib, tile_max, lse, n_valid_rows, c.size(0), e.size(1), float(filter_eps), e.dtype, dev):
+            de_dense, dc_dense, dz_budget = want_de, (want_dc or want_dbias), auto_budget
+    de_sparse = want_de and not de_dense
+    dc_sparse = (want_dc or want_dbias) and not dc_dense
+
+    # Every kernel accumulates in fp32 registers and writes an element of dC and dBias once; dE is written once by
+    # the ownership kernels and carried from chunk to chunk with a 16-bit compensation term by the unfiltered path.
+    # Gradient buffers in fp32 (what accum_e_fp32 / accum_c_fp32 ask the reference for, cce_backward.py:390-394)
+    # would hold the same values before the final cast, so the buffers take the dtype the caller gets back.
+    de_dtype = torch.float32 if e_info.dtype == torch.float32 else e.dtype
+    dc_dtype = torch.float32 if c_info.dtype == torch.float32 else c.dtype
     de = None
-    if e_info.requires_grad:
+    if want_de:
         # the unfiltered path writes every valid row of a 16-bit dE; rows outside `valids` and every other case
         # (the ownership kernels, an fp32 accumulator) start from zeros
-        de_written_whole = dense and valids is None and de_dtype != torch.float32 and n_valid_rows > 0
+        de_written_whole = de_dense and valids is None and de_dtype != torch.float32 and n_valid_rows > 0
         de = torch.empty_like(e, dtype=de_dtype) if de_written_whole else torch.zeros_like(e, dtype=de_dtype)
     dc = None
-    if c_info.requires_grad:
+    if want_dc:
         # both paths write every element of dC (the ownership kernel stores zeros for a class group nothing
         # survived for); only with no valid row at all is nothing launched
         dc = torch.empty_like(c, dtype=dc_dtype) if n_valid_rows > 0 else torch.zeros_like(c, dtype=dc_dtype)
@@ -285,16 +335,7 @@ def cce_backward_kernel(
         assert counters.dtype in (torch.int64, torch.uint64) and counters.numel() >= _hip.NUM_COUNTERS
         assert counters.is_contiguous() and counters.device == dev
 
-    wanted = de is not None or dc is not None or dbias is not None
-    if B > 0 and wanted and dense:
-        _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets, de, dc, dbias, B, grad_scale,
-                        shift, target_offset, softcap)
-        if counters is not None:  # every 32 x 32 sub-tile is recomputed and enters both products
-            tiles = ((B + 31) // 32) * ((c.size(0) + 31) // 32)
-            counters.view(torch.int64)[:4] += torch.tensor(
-                [tiles, tiles, tiles if de is not None else 0, tiles if dc is not None or dbias is not None else 0],
-                dtype=torch.int64, device=dev)
-    elif B > 0 and wanted:
+    if B > 0 and (de_sparse or dc_sparse):
         ws_bytes = lib.cce_backward_workspace_bytes(B, c.size(0), e.size(1))
         workspace = torch.empty((max(ws_bytes, 8) // 8 + 1,), dtype=torch.int64, device=dev)
         with torch.cuda.device(dev), _hip.timed("backward_sparse", dev):
@@ -303,7 +344,8 @@ def cce_backward_kernel(
                 lse.data_ptr(), do.data_ptr(), 1 if do.numel() == 1 else 0, _hip.ptr(dlse),
                 _hip.ptr(valids), _hip.ptr(vocab_ordering), targets.data_ptr(),
                 _hip.ptr(tile_max),
-                _hip.ptr(de), _hip.ptr(dc), _hip.ptr(dbias),
+                _hip.ptr(de if de_sparse else None), _hip.ptr(dc if dc_sparse else None),
+                _hip.ptr(dbias if dc_sparse else None),
                 workspace.data_ptr(), workspace.numel() * 8, _hip.ptr(counters),
                 e.size(0), B, c.size(0), e.size(1),
                 e.stride(0), c.stride(0), c.stride(1),
@@ -315,6 +357,23 @@ def cce_backward_kernel(
                 _hip.current_stream_ptr(dev),
             )
         _hip.check(status, "cce_backward")
+    if B > 0 and (de_dense or dc_dense):
+        _dense_backward(lib, code, dev, e, c, bias, lse, do, dlse, valids, targets,
+                        de if de_dense else None, dc if dc_dense else None, dbias if dc_dense else None,
+                        B, grad_scale, shift, target_offset, softcap, dz_budget)
+        if counters is not None:
+            # every 32 x 32 sub-tile is recomputed (once: a recompute the ownership kernels did for the other
+            # side of a one-sided preset is on top and not counted) and enters the products of this call
+            tiles = ((B + 31) // 32) * ((c.size(0) + 31) // 32)
+            sparse_too = de_sparse or dc_sparse
+            view = counters.view(torch.int64)
+            if sparse_too:
+                view[1] = view[0]  # recomputed = the whole plane, whatever the ownership kernels added
+                view[2:4] += torch.tensor([tiles if de_dense else 0, tiles if dc_dense else 0],
+                                          dtype=torch.int64, device=dev)
+            else:
+                view[:4] += torch.tensor([tiles, tiles, tiles if de_dense else 0, tiles if dc_dense else 0],
+                                         dtype=torch.int64, device=dev)
 
     if dbias is not None:
         assert bias_info is not None

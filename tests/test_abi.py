@@ -29,7 +29,7 @@ def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for want in ("cce_version", "cce_error_string", "cce_tile_stat_elems", "cce_lse_forward_workspace_bytes",
                  "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward",
-                 "cce_backward_dz", "cce_lse_forward_static", "cce_backward_dense",
+                 "cce_backward_dz", "cce_lse_forward_static", "cce_lse_forward_static_init", "cce_backward_dense",
                  "cce_backward_dense_workspace_bytes", "cce_count_flagged_cells", "cce_backward_products"):
         assert want in names
 

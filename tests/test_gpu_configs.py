@@ -272,6 +272,50 @@ def test_config2_full_size_forward_and_backward(monkeypatch):
     assert recomputed / total < 0.05 and with_de / total < 0.02 and with_dc == with_de
 
 
+def test_config2_full_size_one_sided_presets_and_kahan(monkeypatch):
+    """The presets that filter one gradient only (cce_kahan_full_c: dC exact, dE filtered; cce_kahan_full_e: the
+    other way round) and cce_kahan (both filtered, fp32 accumulation asked for) at the headline shape, every element
+    of dE and dC against the dense fp32 oracle with the filter rule on the filtered output only.  cce_kahan must
+    also keep the 16 MB of the filtered path: no fp32 copy of dC is taken for the accumulation flags."""
+    import cut_cross_entropy.cce_backward as bw
+    from cut_cross_entropy import _hip
+    from cut_cross_entropy import linear_cross_entropy
+
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "sparse")
+    N, D, V, softcap = 8192, 2304, 256000, 30.0
+    g = torch.Generator(device=DEV).manual_seed(0)
+    e = torch.randn((N, D), generator=g, device=DEV).to(torch.bfloat16)
+    c = (torch.randn((V, D), generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (N,), generator=g, device=DEV)
+    d_out = torch.full((N,), 1.0 / N, device=DEV)
+    refs = {True: _reference_gradients(e, c, t, None, d_out, None, softcap, filter_eps=2.0**-12),
+            False: _reference_gradients(e, c, t, None, d_out, None, softcap, filter_eps=None)}
+    ed = e.clone().requires_grad_(True)
+    cd = c.clone().requires_grad_(True)
+    for impl, e_filtered, c_filtered, want_paths in (
+            ("cce_kahan_full_c", True, False, ["backward_dense", "backward_sparse"]),
+            ("cce_kahan_full_e", False, True, ["backward_dense", "backward_sparse"]),
+            ("cce_kahan", True, True, ["backward_sparse"])):
+        print("impl", impl, flush=True)
+        ed.grad = cd.grad = None
+        timers = {}
+        _hip.set_timers(timers)
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        loss = linear_cross_entropy(ed, cd, t, softcap=softcap, impl=impl)
+        loss.backward()
+        torch.cuda.synchronize()
+        _hip.set_timers(None)
+        extra_mb = (torch.cuda.max_memory_allocated() - base - ed.grad.numel() * 2 - cd.grad.numel() * 2) / 2**20
+        assert sorted(k for k in timers if k.startswith("backward")) == want_paths
+        if impl == "cce_kahan":
+            assert extra_mb <= 16.0, extra_mb
+        re_, rc_ = refs[e_filtered], refs[c_filtered]
+        _assert_per_element(ed.grad, re_["de_gt"], re_["de_ref"], re_["de_amb"], impl + " dE")
+        _assert_per_element(cd.grad, rc_["dc_gt"], rc_["dc_ref"], rc_["dc_amb"], impl + " dC")
+
+
 @pytest.mark.parametrize("filter_eps", ["auto", None])
 def test_config2_scaled_filter_vs_exact(filter_eps):
     """Near-uniform soft-max: with filtering only the target sub-tiles survive, and the result stays

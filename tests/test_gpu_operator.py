@@ -216,10 +216,10 @@ def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids
 
 def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     """Near-uniform soft-max over few classes: every cell's bound exp(max logit - min lse) is above
-    filter_eps, so the backward runs unfiltered (and is then exact) -- from the second step on: the count of
-    flagged cells is read without waiting for the device, so a step uses the count of the step before, and the
-    first step of a shape runs the ownership kernels.  With the switch off the ownership kernels run.  Peaked
-    soft-max over many classes: the sparse kernels stay."""
+    filter_eps, so the backward runs unfiltered (and is then exact) -- from the FIRST step on: the first backward
+    of a shape waits for the count of its own flagged cells, every later one uses the count of the backward
+    before it, so the same inputs take the same path and give the same bits on every call.  With the switch off
+    the ownership kernels run.  Peaked soft-max over many classes: the sparse kernels stay."""
     from cut_cross_entropy import cce_backward as bw
     from cut_cross_entropy import linear_cross_entropy
     from oracle import dense_lce
@@ -227,20 +227,25 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     calls = []
     real = bw._dense_backward
     monkeypatch.setattr(bw, "_dense_backward", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
-    monkeypatch.setattr(bw, "_monitors", {})
+    bw.reset_backward_path_memory()
 
     e, c, t, _ = make_inputs(512, 2048, 128, torch.bfloat16, seed=4, planted=False, c_std=0.05)
     ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
     e64, c64 = e.double().requires_grad_(True), c.double().requires_grad_(True)
     dense_lce.dense_linear_cross_entropy(e64, c64, t)[0].backward()
-    for step in range(2):
+    first = None
+    for step in range(3):
         ed.grad = cd.grad = None
         linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
         torch.cuda.synchronize()
-        assert len(calls) == step  # step 0: no count yet -> ownership kernels; step 1: dense
-        tol = 2e-2 if step == 1 else 5e-2  # the filtered gradient of step 0 differs by the dropped sub-tiles
-        assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=tol / 512, rtol=tol)
-        assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=tol / 512, rtol=tol)
+        assert len(calls) == step + 1  # dense from the first step on
+        assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=2e-2 / 512, rtol=2e-2)
+        assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=2e-2 / 512, rtol=2e-2)
+        if first is None:
+            first = (ed.grad.clone(), cd.grad.clone())
+        assert torch.equal(ed.grad, first[0]) and torch.equal(cd.grad, first[1])  # call 1 == call n, bit for bit
+    calls.clear()
+    calls.append(1)
 
     monkeypatch.setattr(bw, "DENSE_WHEN_FLAGGED_ABOVE", None)
     ed.grad = cd.grad = None
@@ -259,10 +264,18 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
     assert len(calls) == 2
-    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 64 << 20)
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 1 << 20)
+    ed.grad = cd.grad = None
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
     assert len(calls) == 3
+    # the path the filtered preset took by itself stays inside the limit (dz chunk + compensation buffer + the
+    # forward's small vectors), whatever DENSE_DZ_BYTES would have allowed
+    extra = torch.cuda.max_memory_allocated() - base - ed.grad.numel() * 2 - cd.grad.numel() * 2
+    assert extra <= (1 << 20) + (256 << 10), extra
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", None)
 
     g = torch.Generator().manual_seed(1)
@@ -297,7 +310,73 @@ def test_backward_never_waits_for_the_device(impl):
     assert torch.isfinite(ed.grad).all() and torch.isfinite(cd.grad).all()
 
 
-@pytest.mark.parametrize("impl,path", [("cce", "sparse"), ("cce", "dense"), ("cce_exact", "auto")])
+@pytest.mark.parametrize("impl", ["cce_kahan_full_c", "cce_kahan_full_e"])
+def test_one_sided_presets_split_between_the_two_backward_paths(monkeypatch, impl):
+    """A preset that filters one gradient only runs the filtered side on the ownership kernels and the unfiltered
+    side on the dense path (the reference decides per side inside one kernel, cce_backward.py:211-216): the
+    unfiltered side is the exact gradient, the filtered side the filtered one."""
+    from cut_cross_entropy import _hip
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "sparse")
+    # peaked soft-max: filtering drops most of the plane, so the two sides differ visibly
+    e, c, t, _ = make_inputs(512, 4096, 128, torch.bfloat16, seed=8, planted=True)
+    ed, cd, td = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True), t.cuda()
+
+    def grads(which):
+        ed.grad = cd.grad = None
+        timers = {}
+        _hip.set_timers(timers)
+        try:
+            linear_cross_entropy(ed, cd, td, softcap=20.0, impl=which).backward()
+        finally:
+            _hip.set_timers(None)
+        torch.cuda.synchronize()
+        return ed.grad.clone(), cd.grad.clone(), sorted(k for k in timers if k.startswith("backward"))
+
+    de_f, dc_f, ran_f = grads("cce")
+    de_x, dc_x, ran_x = grads("cce_exact")
+    de_m, dc_m, ran_m = grads(impl)
+    assert ran_f == ["backward_sparse"] and ran_x == ["backward_dense"]
+    assert ran_m == ["backward_dense", "backward_sparse"]
+    assert not torch.equal(dc_f, dc_x) and not torch.equal(de_f, de_x)  # the case tells the sides apart
+    if impl == "cce_kahan_full_c":  # dC unfiltered, dE filtered
+        assert torch.equal(dc_m, dc_x) and torch.equal(de_m, de_f)
+    else:
+        assert torch.equal(de_m, de_x) and torch.equal(dc_m, dc_f)
+
+
+def test_accumulate_flags_take_no_fp32_gradient_buffers():
+    """accum_e_fp32 / accum_c_fp32 ask the reference for fp32 dE / dC buffers (cce_backward.py:390-394).  The kernels
+    here accumulate in fp32 registers and write an element once, so a buffer in the input type holds the same bits
+    after the final cast: the flags change neither the result nor the memory."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+
+    e, c, t, _ = make_inputs(1024, 16384, 256, torch.bfloat16, seed=9, planted=True)
+    ed, cd, td = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True), t.cuda()
+    out = {}
+    for flags in (False, True):
+        ed.grad = cd.grad = None
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        old = bw.FILTERED_BACKWARD_PATH
+        bw.FILTERED_BACKWARD_PATH = "sparse"
+        try:
+            linear_cross_entropy(ed, cd, td, impl="cce", accum_e_fp32=flags, accum_c_fp32=flags).backward()
+        finally:
+            bw.FILTERED_BACKWARD_PATH = old
+        torch.cuda.synchronize()
+        peak = torch.cuda.max_memory_allocated() - base
+        out[flags] = (ed.grad.clone(), cd.grad.clone(), peak - ed.grad.numel() * 2 - cd.grad.numel() * 2)
+    assert torch.equal(out[False][0], out[True][0]) and torch.equal(out[False][1], out[True][1])
+    assert out[True][2] <= out[False][2] + (1 << 16)  # no fp32 copy of dC (33 MB here) anywhere
+
+
+@pytest.mark.parametrize("impl,path", [("cce", "sparse"), ("cce", "dense"), ("cce", "auto"), ("cce_exact", "auto"),
+                                       ("cce_kahan_full_c", "auto"), ("cce_kahan_full_e", "auto")])
 def test_operator_backward_replays_in_a_hip_graph(monkeypatch, impl, path):
     """loss.backward() of the operator captured in a HIP graph (the forward runs eagerly on the capture stream:
     it reads the number of valid rows on the host, as the reference does) and replayed on new contents of e and

@@ -95,3 +95,48 @@ def test_static_scratch_rejects_shapes_beyond_its_size():
                                     B, B, V, D, D, D, 1, 0.0, 0, torch.cuda.current_stream().cuda_stream)
     assert st == 10005
     assert b"static" in lib.cce_error_string(st)
+
+
+def test_static_entry_replays_in_a_hip_graph_after_init():
+    """The set-up call resolves the device's scratch array, so that a FIRST call of the entry point may fall inside a
+    graph capture; every replay, on new contents and with eager work in between, must equal the eager workspace entry."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    assert lib.cce_lse_forward_static_init() == 0
+    N, V, D = 640, 5000, 128
+    g = torch.Generator().manual_seed(21)
+    e = torch.empty((N, D), dtype=torch.bfloat16, device=dev)
+    c = torch.empty((V, D), dtype=torch.bfloat16, device=dev)
+    lse_graph = torch.empty((N,), dtype=torch.float32, device=dev)
+    tm_graph = torch.empty((lib.cce_tile_stat_elems(N, V),), dtype=torch.float32, device=dev)
+
+    def refill():
+        e.copy_(torch.randn((N, D), generator=g).to(torch.bfloat16))
+        c.copy_((torch.randn((V, D), generator=g) * 0.05).to(torch.bfloat16))
+
+    refill()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = lib.cce_lse_forward_static(
+            e.data_ptr(), c.data_ptr(), None, None, lse_graph.data_ptr(), None, tm_graph.data_ptr(),
+            N, N, V, D, e.stride(0), c.stride(0), c.stride(1), 30.0, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0, lib.cce_error_string(st)
+    ws_bytes = lib.cce_lse_forward_workspace_bytes(N, V, D)
+    ws = torch.empty((ws_bytes // 8 + 1,), dtype=torch.int64, device=dev)
+    for rep in range(3):
+        print("replay", rep, flush=True)
+        refill()
+        lse_graph.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        lse_eager = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+        tm_eager = torch.empty_like(tm_graph)
+        st = lib.cce_lse_forward(
+            e.data_ptr(), c.data_ptr(), None, None, lse_eager.data_ptr(), None, tm_eager.data_ptr(),
+            ws.data_ptr(), ws.numel() * 8, N, N, V, D, e.stride(0), c.stride(0), c.stride(1), 30.0, 0,
+            torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.cce_error_string(st)
+        torch.cuda.synchronize()
+        assert torch.isfinite(lse_graph).all()
+        assert torch.equal(lse_graph, lse_eager)
+        assert torch.equal(tm_graph, tm_eager)
