@@ -150,6 +150,26 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Maximum over the 64 lanes as a wave-uniform value, on the vector unit alone: four rotations inside the rows of 16
+// lanes (after which every lane holds its row's maximum), then lane 15 of rows 0 and 2 broadcast into rows 1 and 3
+// and lane 31 into rows 2 and 3; the last lane then holds the maximum of all.  The shuffles of wave_max() above
+// go through the LDS crossbar (one ds_bpermute and a wait each).
+__device__ __forceinline__ float wave_max_uniform(float v) {
+  auto dpp = [](float x, auto ctrl, auto row_mask) {
+    const int r = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                              decltype(row_mask)::value, 0xf, false);
+    return __builtin_bit_cast(float, r);
+  };
+  using std::integral_constant;
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x121>{}, integral_constant<int, 0xf>{}));  // row_ror:1
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x122>{}, integral_constant<int, 0xf>{}));  // row_ror:2
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x124>{}, integral_constant<int, 0xf>{}));  // row_ror:4
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x128>{}, integral_constant<int, 0xf>{}));  // row_ror:8
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{}));  // row_bcast:15 into rows 1, 3
+  v = fmaxf(v, dpp(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{}));  // row_bcast:31 into rows 2, 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 __device__ __forceinline__ float wave_min(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = fminf(v, __shfl_xor(v, off, 64));

@@ -431,6 +431,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
 #pragma unroll
   for (int ti = 0; ti < kF16WT; ++ti) s_run[ti * kFwdThreads] = make_float2(-INFINITY, 0.0f);
 
+  float stat = 0.0f;  // statistic cells waiting to be written (see the epilogue)
   int buf = 0;
   set_class_tile(static_cast<int64_t>(vt_begin) * kFwdTile);
   Fast::prefetch(src, smem);
@@ -490,24 +491,30 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
       }
 
       if (p.tile_max != nullptr) {
-        // max over the 32 rows x 32 classes of each statistic cell of this (wave, row pair)
-        int64_t prow = wrow0 + tp * 32;
-        // (the compiler would otherwise form the per-lane address of every cell row before the tile loop and
-        // hold the pairs of registers through the main loop)
-        asm volatile("" : "+s"(prow));
-        float cell[kF16WV / 2];
+        // Maxima over the 32 rows x 32 classes of the four statistic cells of this (wave, row pair): wave-uniform
+        // values, parked in one register across the lanes -- lane 8 k + 4 tp + j holds cell (row pair tp, class
+        // group j) of the k-th tile of a run of eight -- and written out once per eight tiles: a store after every
+        // tile would have the next tile's first wait for its loads wait for the store's acknowledgement as well.
+        const int slot = (vt - vt_begin) & 7;
 #pragma unroll
-        for (int j = 0; j < kF16WV / 2; ++j) cell[j] = wave_max(bm[j]);
-        if (lane < kF16WV / 2 && prow < p.b && vw0 + lane * 32 < p.v) {
-          float mine = cell[0];
-#pragma unroll
-          for (int j = 1; j < kF16WV / 2; ++j) mine = (lane == j) ? cell[j] : mine;
-          if (fixed_ref) {  // the maximum was taken over raw logits
-            const float t = __builtin_amdgcn_exp2f(mine * p.sc.in_scale);
-            mine = fmaf(__builtin_amdgcn_rcpf(1.0f + t), -2.0f * p.sc.out_scale, p.sc.out_scale);
-          }
-          p.tile_max[(prow / CCE_STAT_ROWS) * p.stat_cols + vw0 / CCE_STAT_COLS + lane] = mine * kLn2;
+        for (int j = 0; j < kF16WV / 2; ++j) {
+          const float cell = wave_max_uniform(bm[j]);
+          stat = (lane == 8 * slot + 4 * tp + j) ? cell : stat;
         }
+      }
+    }
+    if (p.tile_max != nullptr && (((vt - vt_begin) & 7) == 7 || vt + 1 == vt_end)) {
+      const int first_vt = vt - ((vt - vt_begin) & 7);
+      const int my_vt = first_vt + (lane >> 3);
+      const int64_t row = wrow0 + ((lane >> 2) & 1) * 32;
+      const int64_t cls = static_cast<int64_t>(my_vt) * kFwdTile + wv * (16 * kF16WV) + (lane & 3) * 32;
+      if (my_vt <= vt && row < p.b && cls < p.v) {
+        float mine = stat;
+        if (fixed_ref) {  // the maximum was taken over raw logits
+          const float t = __builtin_amdgcn_exp2f(mine * p.sc.in_scale);
+          mine = fmaf(__builtin_amdgcn_rcpf(1.0f + t), -2.0f * p.sc.out_scale, p.sc.out_scale);
+        }
+        p.tile_max[(row / CCE_STAT_ROWS) * p.stat_cols + cls / CCE_STAT_COLS] = mine * kLn2;
       }
     }
   }
