@@ -624,7 +624,10 @@ struct DmaLogitTile16 {
   static constexpr int load_slot(int j) { return j < 6 ? kSyncAt + 2 + 4 * j : kSlots - 4 + 2 * (j - 6); }
   static_assert(WV == 8 && WT == 4 && NQ == 8, "the slot tables above are laid out for 8 x 4 blocks and 8 loads");
 
-  template <bool READ, bool LOAD, bool SYNC>
+  // ZERO (the first step of a tile): the accumulators start from the instruction's constant zero instead of being
+  // cleared beforehand (128 register writes per lane and tile; the copy of the first stage this takes costs a
+  // cool chip with idle operands 3 %, and gains 2 % under real operands, where the chip is power-bound).
+  template <bool READ, bool LOAD, bool SYNC, bool ZERO = false>
   static __device__ __forceinline__ void step(f32x4 (&acc)[WV][WT], vec8 (&a)[WV], const vec8 (&bc)[WT], vec8 (&bn)[WT],
                                               const unsigned char* rd_c, const unsigned char* rd_e, const Source& src,
                                               int koff, unsigned lds_base, int ld_stage, int wave) {
@@ -635,7 +638,7 @@ struct DmaLogitTile16 {
         wait_vmcnt<0>();
         __syncthreads();
       }
-      acc[vi][ti] = Elem<T>::mfma16(a[vi], bc[ti], acc[vi][ti]);
+      acc[vi][ti] = Elem<T>::mfma16(a[vi], bc[ti], ZERO ? f32x4{0.0f, 0.0f, 0.0f, 0.0f} : acc[vi][ti]);
       __builtin_amdgcn_sched_barrier(0);
       if (READ) {
         static_for<WT>([&](auto t_c) {
@@ -668,13 +671,14 @@ struct DmaLogitTile16 {
   }
 
   // D must be a multiple of 64 and at least 128.  The first two stages of this tile must be in flight or landed in
-  // ring stages buf, 1 - buf (prefetch(), or the previous run()), and nothing else may have touched the ring.
+  // ring stages buf, 1 - buf (prefetch() for the first tile of a span: first_tile; else the previous run()), and
+  // nothing else may have touched the ring.
   // next_tile() is called once, when the class rows of this tile have been fetched for the last time: it points
   // `src` at the tile whose first stages the rest of this run fetches (or leaves it: those loads then repeat this
   // tile's first stages and are never read).
   template <typename NextTile>
   static __device__ __forceinline__ void run(f32x4 (&acc)[WV][WT], Source& src, unsigned char* lds, int D, int& buf,
-                                             NextTile&& next_tile) {
+                                             bool first_tile, NextTile&& next_tile) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wv = wave / NWT;
@@ -688,25 +692,31 @@ struct DmaLogitTile16 {
     const unsigned char* e_row = lds + (TILE_V + wt * WT * 16 + r16) * kDmaRowBytes;
     const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
 
-#pragma unroll
-    for (int vi = 0; vi < WV; ++vi)
-#pragma unroll
-      for (int ti = 0; ti < WT; ++ti)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[vi][ti][r] = 0.0f;
-
     const int nk = D / kDmaBK;
     int cur = buf * STAGE_BYTES;
-    wait_vmcnt<NQ>();  // the first stage has landed, the second may be in flight
-    __syncthreads();
+    if (first_tile) {
+      wait_vmcnt<NQ>();  // the first stage has landed for this wave (the second may be in flight) ...
+      __syncthreads();   // ... and for all of them
+    }
+    // (a later tile's first stage was awaited by every wave before the last barrier of the tile before it: no
+    // barrier here, so a wave that leaves its epilogue early starts on the next tile while the others finish)
     vec8 a[WV], b0[WT], b1[WT];
 #pragma unroll
     for (int ti = 0; ti < WT; ++ti) b0[ti] = frag(e_row + cur + chunk0 + ti * 16 * kDmaRowBytes);
 #pragma unroll
     for (int vi = 0; vi < WV; ++vi) a[vi] = frag(c_row + cur + chunk0 + vi * 16 * kDmaRowBytes);
 
+    // first stage (never the last: D >= 128)
+    {
+      const int nxt = STAGE_BYTES - cur;
+      step<true, false, false, true>(acc, a, b0, b1, c_row + cur + chunk1, e_row + cur + chunk1, src, 0, lds_base, 0, wave);
+      if (nk == 2) next_tile();
+      step<true, true, true>(acc, a, b1, b0, c_row + nxt + chunk0, e_row + nxt + chunk0, src, (2 < nk) ? 2 * kDmaBK : 0,
+                             lds_base, cur, wave);
+      cur = nxt;
+    }
 #pragma unroll 1
-    for (int s = 0; s < nk - 1; ++s) {
+    for (int s = 1; s < nk - 1; ++s) {
       const int nxt = STAGE_BYTES - cur;
       step<true, false, false>(acc, a, b0, b1, c_row + cur + chunk1, e_row + cur + chunk1, src, 0, lds_base, 0, wave);
       if (s == nk - 2) next_tile();

@@ -450,7 +450,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
       }
     }
     f32x4 acc[kF16WV][kF16WT];
-    Fast::run(acc, src, smem, static_cast<int>(p.d), buf, [&] {
+    Fast::run(acc, src, smem, static_cast<int>(p.d), buf, vt == vt_begin, [&] {
       if (vt + 1 < vt_end) set_class_tile(v0 + kFwdTile);
     });
 
