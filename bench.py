@@ -174,6 +174,36 @@ def cpu_baseline(w, rows):
     }
 
 
+def gemm_yardstick(args, w, e2, c):
+    """The library's matrix product of the forward's shape, timed with device events like the forward kernel."""
+    import torch
+
+    n, d = e2.shape
+    v = c.shape[0]
+    out = torch.empty((n, v), dtype=e2.dtype, device=e2.device)
+    for _ in range(args.warmup):
+        torch.mm(e2, c.t(), out=out)
+    torch.cuda.synchronize()
+    evs = []
+    for _ in range(args.steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        torch.mm(e2, c.t(), out=out)
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    peak = PEAK_FP32_TFLOPS if args.dtype == "fp32" else PEAK_BF16_TFLOPS
+    tflops = 2.0 * n * v * d / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "library matrix product E . C^T (yardstick, not the loss path)",
+        "config": {"workload": f"{w['name']}: E[{n},{d}] x C[{v},{d}]^T {args.dtype} -> [{n},{v}] {args.dtype}, torch.mm "
+                               f"(hipBLASLt / rocBLAS), {w['text']}"},
+        "steps": args.steps, "warmup": args.warmup, "ms_per_launch": ms, "tflops": tflops, "frac": tflops / peak,
+        "peak": peak, "output_bytes": out.numel() * out.element_size(),
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -189,6 +219,12 @@ def main():
     ap.add_argument("--dense-workspace-mb", type=float, default=None,
                     help="cap the workspace of the unfiltered backward (dz chunk + dE compensation buffer) at this "
                          "many MB, for presets that ask for it and for a filtered backward that changes to it")
+    ap.add_argument("--zero-data", action="store_true",
+                    help="run the workload's shapes on operands of zeros: the kernels do the same work at the clock "
+                         "the chip holds when the matrix pipes toggle nothing (what the power limit costs)")
+    ap.add_argument("--gemm-yardstick", action="store_true",
+                    help="instead of the loss path, time the library's plain matrix product E . C^T of the workload's "
+                         "shape and input type (the logits the forward kernel never writes), and print its TFLOP/s")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--traffic-probe", action="store_true",
@@ -223,9 +259,16 @@ def main():
         bwd_mod.DENSE_DZ_BYTES = max(limit - comp, 0)
         bwd_mod.DENSE_DZ_MIN_CLASSES = 0
     in_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
+    if args.zero_data:
+        w["e"].zero_()
+        w["c"].zero_()
+        w["text"] += " [operands replaced by zeros]"
     e = w["e"].to(dev).to(in_dtype).requires_grad_(True)
     c = w["c"].to(dev).to(in_dtype).requires_grad_(True)
     t = w["t"].to(dev)
+    if args.gemm_yardstick:
+        gemm_yardstick(args, w, e.detach().reshape(-1, w["D"]), c.detach())
+        return
     bias = None
     if args.bias:
         gb = torch.Generator().manual_seed(1)

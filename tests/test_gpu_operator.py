@@ -310,6 +310,32 @@ def test_backward_never_waits_for_the_device(impl):
     assert torch.isfinite(ed.grad).all() and torch.isfinite(cd.grad).all()
 
 
+def test_a_width_that_is_no_multiple_of_128_costs_padded_copies_and_nothing_else(monkeypatch):
+    """D = 200 runs the direct-to-LDS kernels on copies of e and c padded to 256 columns (one copy each in the
+    forward, the padded dC and the slice back in the backward).  The copies are the whole price: the loss path's
+    transient memory stays below the padded copies plus the padded gradient, and the results match an aligned run
+    of the same numbers."""
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+
+    monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "sparse")
+    N, V, D, Dp = 512, 8192, 200, 256
+    e, c, t, _ = make_inputs(N, V, D, torch.bfloat16, seed=13, planted=True)
+    ed, cd, td = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True), t.cuda()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    linear_cross_entropy(ed, cd, td, softcap=20.0, impl="cce").backward()
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated() - base - (ed.grad.numel() + cd.grad.numel()) * 2
+    padded = (N + V) * Dp * 2
+    assert extra <= 2 * padded + (4 << 20), (extra, padded)  # padded e and c, padded dE and dC, small vectors
+    ep = torch.nn.functional.pad(e, (0, Dp - D)).cuda().requires_grad_(True)
+    cp = torch.nn.functional.pad(c, (0, Dp - D)).cuda().requires_grad_(True)
+    linear_cross_entropy(ep, cp, td, softcap=20.0, impl="cce").backward()
+    assert torch.equal(ed.grad, ep.grad[:, :D]) and torch.equal(cd.grad, cp.grad[:, :D])
+
+
 @pytest.mark.parametrize("impl", ["cce_kahan_full_c", "cce_kahan_full_e"])
 def test_one_sided_presets_split_between_the_two_backward_paths(monkeypatch, impl):
     """A preset that filters one gradient only runs the filtered side on the ownership kernels and the unfiltered
