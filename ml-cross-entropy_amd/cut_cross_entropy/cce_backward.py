@@ -56,6 +56,7 @@ FILTERED_BACKWARD_PATH = "auto"
 # (cce_exact, cce_kahan_full_*) are not bound by it: their dz chunk is DENSE_DZ_BYTES (the reference's own
 # unfiltered presets take fp32 copies of dE and dC, 2.3 GB at E [8192, 2304] x C [256000, 2304]).
 DENSE_WORKSPACE_LIMIT_BYTES: Optional[int] = 256 << 20
+AUTO_DENSE_MIN_CLASSES = 1024
 _OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
 
@@ -101,16 +102,19 @@ def reset_backward_path_memory() -> None:
 
 def _auto_dense_dz_budget(lib, B: int, V: int, D: int, de_16bit: bool) -> Optional[int]:
     """dz chunk bytes a filtered backward may use when it changes to the unfiltered path by itself, or None when
-    even the smallest plan exceeds DENSE_WORKSPACE_LIMIT_BYTES."""
+    DENSE_WORKSPACE_LIMIT_BYTES leaves no room for chunks of a useful size."""
     budget = _dz_budget(B)
     if DENSE_WORKSPACE_LIMIT_BYTES is None:
         return budget
     comp = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0) - \
         lib.cce_backward_dense_workspace_bytes(B, V, D, 0, 0)
-    smallest = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0)
-    if smallest > DENSE_WORKSPACE_LIMIT_BYTES:
+    # Chunks of fewer than AUTO_DENSE_MIN_CLASSES classes are not worth having: every chunk passes over all of dE, and
+    # its products reduce over a handful of stages (measured, backward of E [15356, 4096] x C [128256, 4096]: 226 ms
+    # with 256 classes per chunk, 45 ms with 2048, 39 ms with 8192, against 168 ms on the ownership kernels).
+    room = DENSE_WORKSPACE_LIMIT_BYTES - comp
+    if room < 2 * B * min(AUTO_DENSE_MIN_CLASSES, (V + 255) // 256 * 256):
         return None
-    return min(budget, DENSE_WORKSPACE_LIMIT_BYTES - comp)
+    return min(budget, room)
 
 
 def _filtered_backward_runs_dense(lib, tile_max, lse, B: int, V: int, D: int, filter_eps: float, dtype, dev) -> bool:

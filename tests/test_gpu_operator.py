@@ -264,7 +264,12 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
     assert len(calls) == 2
+    # (1 MB would leave room for 896 of the 1024 classes a chunk must hold at least: the ownership kernels again)
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 1 << 20)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 2
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 2 << 20)
     ed.grad = cd.grad = None
     torch.cuda.synchronize()
     base = torch.cuda.memory_allocated()
@@ -275,7 +280,7 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     # the path the filtered preset took by itself stays inside the limit (dz chunk + compensation buffer + the
     # forward's small vectors), whatever DENSE_DZ_BYTES would have allowed
     extra = torch.cuda.max_memory_allocated() - base - ed.grad.numel() * 2 - cd.grad.numel() * 2
-    assert extra <= (1 << 20) + (256 << 10), extra
+    assert extra <= (2 << 20) + (256 << 10), extra
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", None)
 
     g = torch.Generator().manual_seed(1)
