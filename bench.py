@@ -256,6 +256,7 @@ def main():
         limit = int(args.dense_workspace_mb * 2**20)
         comp = 2 * w["valid"] * w["D"]  # the 16-bit compensation buffer of dE
         bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES = limit
+        bwd_mod.DENSE_WORKSPACE_LIMIT_OPERANDS = 0.0
         bwd_mod.DENSE_DZ_BYTES = max(limit - comp, 0)
         bwd_mod.DENSE_DZ_MIN_CLASSES = 0
     in_dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
@@ -365,7 +366,8 @@ def main():
             "valid_tokens": B,
             "impl": w["impl"],
             "dense_workspace_limit_mb": None if bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES is None
-            else bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES / 2**20,
+            else max(bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES,
+                     bwd_mod.DENSE_WORKSPACE_LIMIT_OPERANDS * (B * D + V * D) * in_dtype.itemsize) / 2**20,
         },
         "loss": float(loss),
         "loss_path_peak_mb": extra_mb,
@@ -374,9 +376,9 @@ def main():
         "fwd_bwd_frac_alg": f_alg / (ms_per_step * 1e-3) / 1e12 / peak,
         "fwd_bwd_frac_dense_equiv": f_dense / (ms_per_step * 1e-3) / 1e12 / peak,
         "roofline": {
-            "kernel": ("the fp32 forward (three-way bf16 split of e and c, lse_forward_kernel per vocabulary chunk, merge)"
+            "kernel": ("the fp32 forward (three-way bf16 split of e and c, lse_forward16_kernel per vocabulary chunk, merge)"
                        if args.dtype == "fp32" else
-                       "lse_forward_kernel (fused E.C^T + softcap + online log-sum-exp)")
+                       "lse_forward16_kernel (fused E.C^T + softcap + online log-sum-exp)")
                       + ", device events around its launches inside the timed steps",
             "bound": "mfma",
             "achieved": fwd_tflops,

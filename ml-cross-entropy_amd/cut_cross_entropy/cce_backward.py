@@ -48,14 +48,20 @@ def _dz_budget(B: int) -> int:
 # and the graph replays that path.  FILTERED_BACKWARD_PATH pins the choice: "sparse" or "dense" instead of "auto".
 DENSE_WHEN_FLAGGED_ABOVE = 0.17
 FILTERED_BACKWARD_PATH = "auto"
-# A filtered backward that changes to the unfiltered path BY ITSELF may take at most this much workspace (the dz
-# chunk, plus the [B, D] 16-bit compensation buffer of dE): the ownership kernels need well under 16 MB, and a
-# caller who picked a filtered preset did not ask for more.  The dz chunk shrinks to fit (more, smaller chunks:
-# slower); if not even the smallest plan fits -- the compensation buffer alone can exceed it when rows are many --
-# the backward stays on the ownership kernels.  None: no limit.  The presets that ask for unfiltered gradients
-# (cce_exact, cce_kahan_full_*) are not bound by it: their dz chunk is DENSE_DZ_BYTES (the reference's own
+# A filtered backward that changes to the unfiltered path BY ITSELF may take at most
+#     max(DENSE_WORKSPACE_LIMIT_BYTES, DENSE_WORKSPACE_LIMIT_OPERANDS x (bytes of E + bytes of C))
+# of workspace (the dz chunk, plus the [B, D] 16-bit compensation buffer of dE): the ownership kernels need well
+# under 16 MB, and a caller who picked a filtered preset did not ask for more.  The defaults, 256 MB and 1.0, say:
+# never more than the operands the caller already holds take themselves, and 256 MB where they are smaller (the
+# second term matters when rows are many: at E [65536, 3584] x C [19008, 3584] the compensation buffer alone is
+# 448 MB and the operands are 578 MB; the ownership kernels take 167 ms there, the unfiltered path 22 - 30).  The dz chunk
+# shrinks to fit (more, smaller chunks: slower); if no plan with chunks of AUTO_DENSE_MIN_CLASSES classes fits, the
+# backward stays on the ownership kernels.  DENSE_WORKSPACE_LIMIT_BYTES = None: no limit;
+# DENSE_WORKSPACE_LIMIT_OPERANDS = 0: the byte limit alone.  The presets that ask for unfiltered gradients
+# (cce_exact, cce_kahan_full_*) are not bound by either: their dz chunk is DENSE_DZ_BYTES (the reference's own
 # unfiltered presets take fp32 copies of dE and dC, 2.3 GB at E [8192, 2304] x C [256000, 2304]).
 DENSE_WORKSPACE_LIMIT_BYTES: Optional[int] = 256 << 20
+DENSE_WORKSPACE_LIMIT_OPERANDS: float = 1.0
 AUTO_DENSE_MIN_CLASSES = 1024
 _OWNERSHIP_SLICE_COLS = 2304  # columns of D one ownership workgroup accumulates
 
@@ -100,18 +106,19 @@ def reset_backward_path_memory() -> None:
         _monitors.clear()
 
 
-def _auto_dense_dz_budget(lib, B: int, V: int, D: int, de_16bit: bool) -> Optional[int]:
+def _auto_dense_dz_budget(lib, B: int, V: int, D: int, de_16bit: bool, operand_bytes: int) -> Optional[int]:
     """dz chunk bytes a filtered backward may use when it changes to the unfiltered path by itself, or None when
-    DENSE_WORKSPACE_LIMIT_BYTES leaves no room for chunks of a useful size."""
+    the workspace limit leaves no room for chunks of a useful size."""
     budget = _dz_budget(B)
     if DENSE_WORKSPACE_LIMIT_BYTES is None:
         return budget
+    limit = max(int(DENSE_WORKSPACE_LIMIT_BYTES), int(DENSE_WORKSPACE_LIMIT_OPERANDS * operand_bytes))
     comp = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0) - \
         lib.cce_backward_dense_workspace_bytes(B, V, D, 0, 0)
     # Chunks of fewer than AUTO_DENSE_MIN_CLASSES classes are not worth having: every chunk passes over all of dE, and
     # its products reduce over a handful of stages (measured, backward of E [15356, 4096] x C [128256, 4096]: 226 ms
     # with 256 classes per chunk, 45 ms with 2048, 39 ms with 8192, against 168 ms on the ownership kernels).
-    room = DENSE_WORKSPACE_LIMIT_BYTES - comp
+    room = limit - comp
     if room < 2 * B * min(AUTO_DENSE_MIN_CLASSES, (V + 255) // 256 * 256):
         return None
     return min(budget, room)
@@ -274,7 +281,8 @@ def cce_backward_kernel(
         # ... unless so many cells are flagged that filtering cannot pay: then everything runs unfiltered (exact)
         de_16bit = want_de and e_info.dtype != torch.float32
         auto_budget = dz_budget if (de_dense or dc_dense) else _auto_dense_dz_budget(
-            lib, n_valid_rows, c.size(0), e.size(1), de_16bit)
+            lib, n_valid_rows, c.size(0), e.size(1), de_16bit,
+            n_valid_rows * e.size(1) * e.element_size() + c.numel() * c.element_size())
         if auto_budget is not None and _filtered_backward_runs_dense(
                 lib, tile_max, lse, n_valid_rows, c.size(0), e.size(1), float(filter_eps), e.dtype, dev):
             de_dense, dc_dense, dz_budget = want_de, (want_dc or want_dbias), auto_budget

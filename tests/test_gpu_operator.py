@@ -260,6 +260,7 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     assert len(calls) == 2
     monkeypatch.setattr(bw, "FILTERED_BACKWARD_PATH", "auto")
     # a workspace limit below what the unfiltered path needs here keeps the ownership kernels; above, it does not
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_OPERANDS", 0.0)
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 64 * 1024)
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
@@ -269,6 +270,18 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
     assert len(calls) == 2
+    # the limit is the larger of the byte figure and a multiple of what E and C occupy (here 640 KB): once leaves
+    # 512 KB beside the compensation buffer, twice leaves room for the 1 MB of a 1024-class chunk
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 64 * 1024)
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_OPERANDS", 1.0)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 2
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_OPERANDS", 2.0)
+    linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
+    torch.cuda.synchronize()
+    assert len(calls) == 3
+    monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_OPERANDS", 0.0)
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", 2 << 20)
     ed.grad = cd.grad = None
     torch.cuda.synchronize()
@@ -276,7 +289,7 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     torch.cuda.reset_peak_memory_stats()
     linear_cross_entropy(ed, cd, t.cuda(), impl="cce").backward()
     torch.cuda.synchronize()
-    assert len(calls) == 3
+    assert len(calls) == 4
     # the path the filtered preset took by itself stays inside the limit (dz chunk + compensation buffer + the
     # forward's small vectors), whatever DENSE_DZ_BYTES would have allowed
     extra = torch.cuda.max_memory_allocated() - base - ed.grad.numel() * 2 - cd.grad.numel() * 2
@@ -291,7 +304,7 @@ def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     for _ in range(2):
         linear_cross_entropy(ed2, cd2, t2.cuda(), impl="cce").backward()
         torch.cuda.synchronize()
-    assert len(calls) == 3
+    assert len(calls) == 4
 
 
 @pytest.mark.parametrize("impl", ["cce", "cce_exact"])
