@@ -635,7 +635,8 @@ struct FastLds {
 };
 constexpr int kFLdsBytes = FastLds<false>::kBytes;
 constexpr int kFLightLdsBytes = FastLds<true>::kBytes;
-constexpr int kFLightMaxEntries = 2;                // entries of a class group the light dC pass takes on
+constexpr int kFLightMaxEntries = 2;
+constexpr int kLightStores = 4;                     // store instructions per wave and 128-column chunk of the light dC pass                // entries of a class group the light dC pass takes on
 constexpr int kFSegCells = 512;                     // dE: cells scanned per pass (<= 2048 entries)
 constexpr int kFListCap = 2048;
 static_assert(kFLdsBytes <= 160 * 1024 && 2 * kFLightLdsBytes <= 160 * 1024, "LDS budget of gfx950");
@@ -668,8 +669,9 @@ __device__ __forceinline__ typename Elem<T>::vec8 fstage_frag_transposed(const u
   return __builtin_bit_cast(typename Elem<T>::vec8, v);
 }
 
-// s_waitcnt vmcnt(n) for a wave-uniform n out of the values the ring below can ask for (the immediate
-// must be a constant); anything else waits for everything, which is always safe.
+// s_waitcnt vmcnt(n) for a wave-uniform n out of the values the rings below can ask for (the immediate must be a
+// constant); anything else waits for everything, which is always safe.  The list is kept short: the product loop of
+// the full variant is unrolled 18 times around it.
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
   switch (n) {
     case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
@@ -680,6 +682,17 @@ __device__ __forceinline__ void wait_vmcnt_upto(int n) {
     case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
     case 18: asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); break;
     case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+// ... and for any even n up to 30 (the light variant, whose product loop is not unrolled).
+__device__ __forceinline__ void wait_vmcnt_upto_wide(int n) {
+  switch (n) {
+#define CCE_WAIT_CASE(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    CCE_WAIT_CASE(2) CCE_WAIT_CASE(4) CCE_WAIT_CASE(6) CCE_WAIT_CASE(8) CCE_WAIT_CASE(10) CCE_WAIT_CASE(12)
+    CCE_WAIT_CASE(14) CCE_WAIT_CASE(16) CCE_WAIT_CASE(18) CCE_WAIT_CASE(20) CCE_WAIT_CASE(22) CCE_WAIT_CASE(24)
+    CCE_WAIT_CASE(26) CCE_WAIT_CASE(28) CCE_WAIT_CASE(30)
+#undef CCE_WAIT_CASE
     default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
   }
 }
@@ -779,12 +792,14 @@ __global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_ker
     const int id = own_ids[l32];
     if (id < 0) return;
     uint16_t* dst = static_cast<uint16_t*>(p.d_c) + static_cast<int64_t>(id) * own_sr + d_begin + ci * kFCols + wave * 32 + 4 * half;
+    // exactly kLightStores store instructions per wave and chunk (the product loop below counts them: stores share
+    // the counter its loads are awaited on), whatever the compiler would make of four plain assignments
 #pragma unroll
-    for (int r4 = 0; r4 < 4; ++r4) {
+    for (int r4 = 0; r4 < kLightStores; ++r4) {
       uint2 pk;
       pk.x = Elem<T>::pack2(a[r4 * 4 + 0], a[r4 * 4 + 1]);
       pk.y = Elem<T>::pack2(a[r4 * 4 + 2], a[r4 * 4 + 3]);
-      *reinterpret_cast<uint2*>(dst + 8 * r4) = pk;
+      asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(dst + 8 * r4), "v"(pk) : "memory");
     }
   };
 
@@ -919,23 +934,20 @@ __global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_ker
       // 2 e and 2 e + 1 of a wave belong to entry e), so a short trip moves proportionally less data.
       // A short trip has small stages, so more of them fit the ring and more loads are in flight: a
       // stage holds the rows of the present entries followed by the own rows.
-      const int own_off = 32 * nent * kFRowBytes;
-      const int slot_bytes = own_off + kFOwnBytes;
-      const int ring = Lds::kRing / slot_bytes;  // slots of this size in the ring: 3 / 5 / 7 (light: 2 / 3)
+      // (The logit phase below has its own compile-time geometry: slots of entries + own rows.  The product phase
+      // fetches no own rows, so its slots hold the entries' rows alone and more of them fit the ring: 3 / 5 / 7 / 7
+      // slots for 4 / 3 / 2 / 1 entries, light 3 / 6 for 2 / 1 -- 7 at most, the waits below know no deeper ring.)
+      const int slot_bytes = 32 * nent * kFRowBytes;
+      const int ring = min(7, Lds::kRing / slot_bytes);
       const int ahead = ring - 1;                              // stages in flight
-      // load q of this wave for the stage that starts at column col0: q < 8 other side, q = 8, 9 own side
-      auto issue_load = [&](int q, int col0, int slot, bool with_own, uint32_t entries) {
-        const unsigned base = lds_base + slot * slot_bytes;
-        if (q < 8) {
-          if ((entries >> (q >> 1)) & 1u)
-            lds_dma16(other_ptr[q & 7] + (((other_live >> q) & 1u) ? col0 : 0), base + (q * 4 + wave) * 1024);
-        } else if (with_own) {
-          lds_dma16(own_ptr[q & 1] + (own_step[q & 1] ? col0 : 0), base + own_off + ((q - 8) * 4 + wave) * 1024);
-        }
+      // product phase: load q of this wave (rows of entry q / 2) for the stage that starts at column col0
+      auto issue_load = [&](int q, int col0, int slot, uint32_t entries) {
+        if ((entries >> (q >> 1)) & 1u)
+          lds_dma16(other_ptr[q] + (((other_live >> q) & 1u) ? col0 : 0), lds_base + slot * slot_bytes + (q * 4 + wave) * 1024);
       };
-      auto issue_stage = [&](int col0, int slot, bool with_own, uint32_t entries) {
+      auto issue_stage = [&](int col0, int slot, uint32_t entries) {
 #pragma unroll
-        for (int q = 0; q < 10; ++q) issue_load(q, col0, slot, with_own, entries);
+        for (int q = 0; q < 8; ++q) issue_load(q, col0, slot, entries);
       };
 
       // ---- logits^T of (entry of this wave) x (own rows): 2 nent + 2 loads per wave and stage -----------
@@ -1113,10 +1125,14 @@ __global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_ker
         const int nused = __popc(mask);
         const int npre = min(ahead, nchunks);
 #pragma unroll 1
-        for (int j = 0; j < npre; ++j) issue_stage(d_begin + j * kFCols, j, false, mask);
+        for (int j = 0; j < npre; ++j) issue_stage(d_begin + j * kFCols, j, mask);
         int pslot = 0;  // ci % ring
         auto product_chunk = [&](int ci, f32x16& accum, auto in_agpr) {
-          wait_vmcnt_upto(min(ahead - 1, nchunks - 1 - ci) * 2 * nused);  // the stages after ci may be in flight
+          // The stages after ci may be in flight -- and, in the light variant, the stores of the chunks whose loads
+          // were issued after those of ci (memory operations of a wave complete in issue order and share one counter;
+          // a wait that forgot the stores would wait for the newest loads and for the stores' acknowledgements).
+          if constexpr (LIGHT) wait_vmcnt_upto_wide(min(ahead - 1, nchunks - 1 - ci) * 2 * nused + kLightStores * min(ahead, ci));
+          else wait_vmcnt_upto(min(ahead - 1, nchunks - 1 - ci) * 2 * nused);
           __syncthreads();
           const unsigned char* so = smem + pslot * slot_bytes;
           const int next_col = d_begin + (ci + ahead) * kFCols;
@@ -1133,7 +1149,7 @@ __global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_ker
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const int kk = 4 * h + j;
-              issue_load(kk, next_col, next_slot, false, next_mask);
+              issue_load(kk, next_col, next_slot, next_mask);
               if ((mask >> (kk >> 1)) & 1u) {
                 if constexpr (decltype(in_agpr)::value) Elem<T>::mfma_agpr(a[j], bz[kk], accum);
                 else Elem<T>::mfma_vgpr(a[j], bz[kk], accum);
