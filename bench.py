@@ -254,7 +254,8 @@ def main():
         w["text"] += f" [run with impl={args.impl}]"
     if args.dense_workspace_mb is not None:
         limit = int(args.dense_workspace_mb * 2**20)
-        comp = 2 * w["valid"] * w["D"]  # the 16-bit compensation buffer of dE
+        # the 16-bit compensation buffer of the gradient the unfiltered backward carries between its launches
+        comp = _hip.load().cce_backward_dense_fixed_bytes(w["valid"], w["V"], w["D"], 1)
         bwd_mod.DENSE_WORKSPACE_LIMIT_BYTES = limit
         bwd_mod.DENSE_WORKSPACE_LIMIT_OPERANDS = 0.0
         bwd_mod.DENSE_DZ_BYTES = max(limit - comp, 0)

@@ -214,11 +214,18 @@ int cce_backward_dz(const void* e, const void* c, const void* bias,
                     float grad_scale, int64_t shift, int64_t target_offset,
                     float softcap, int dtype, void* stream);
 
-/* Workspace bytes of cce_backward_dense for a dz chunk buffer of at most `max_dz_bytes` (the function rounds
- * it down to whole 256-class tiles of b rows, at most 16384 classes, and never goes below one tile), plus the
- * 16-bit compensation term of dE, [b, d], when `d_e_in_workspace` (d_e wanted in the 16-bit input type). */
+/* Workspace bytes of cce_backward_dense for a dz buffer of at most `max_dz_bytes` (the function rounds it down to
+ * whole 256-class tiles of b rows, at most 16384 classes -- or, where it walks by rows, to whole 256-row blocks of all
+ * classes -- and never goes below one tile), plus the 16-bit compensation term of the gradient it carries from
+ * launch to launch when `d_e_in_workspace` (d_e wanted in the 16-bit input type): [b, d] for dE, or [v, d] for dC
+ * where b >= 2 v and the walk goes by blocks of rows (see cce_backward_dense).
+ * cce_backward_dense_fixed_bytes is the second part alone; cce_backward_dense_dz_bytes the size of a dz buffer of
+ * `units` classes per chunk (rows per block where the walk goes by rows), for a caller that sizes the workspace
+ * against a limit of its own. */
 int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace,
                                            int64_t max_dz_bytes);
+int64_t cce_backward_dense_fixed_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace);
+int64_t cce_backward_dense_dz_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace, int64_t units);
 
 /*
  * The whole unfiltered backward in one call: d_e, d_c, d_bias of cce_backward with the gradient filter
@@ -240,6 +247,11 @@ int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int 
  *            two differ by the rounding of each term (2^-9 relative for bf16, unbiased)
  *   workspace  256-byte aligned; at least cce_backward_dense_workspace_bytes(b, v, d, d_e in `dtype`, 0) bytes.
  *            Anything beyond that enlarges the chunks (fewer, better filled launches) up to 16384 classes.
+ * With a 16-bit d_e and b >= 2 v (rounded up to 256: a vocabulary shard) the walk goes over blocks of ROWS with the
+ * whole vocabulary each instead: d_e of a block is complete after its launch and written once, and it is d_c that
+ * is carried from block to block (a 16-bit d_c as a pair with a [v, d] compensation term in the workspace, an fp32
+ * d_c in place).  The same number of launches for the same dz buffer, with the smaller matrix as the one that is
+ * read and written once per launch.
  * Layout requirements as for cce_backward_dz (16-byte aligned e, c and d_e, unit stride_cd, row strides that
  * are multiples of 8, d a multiple of 64), else CCE_ERR_MISALIGNED and the caller uses cce_backward.
  */

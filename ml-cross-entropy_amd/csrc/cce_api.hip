@@ -1,7 +1,7 @@
 // Version and status text of the C ABI.
 #include "cce_common.h"
 
-extern "C" int cce_version(void) { return 7; }
+extern "C" int cce_version(void) { return 8; }
 
 #ifndef CCE_SOURCE_HASH
 #define CCE_SOURCE_HASH "unknown"

@@ -14,6 +14,10 @@
 //   3. dense_de_kernel    dE += dz . C[chunk]  : accumulated across the chunks in d_e itself, in fp32 when the caller
 //                         asked for an fp32 dE, else as d_e (16 bit) plus a 16-bit compensation term in the workspace,
 //   4. dz_colsum_kernel   dBias[chunk], when wanted.
+// Where the rows are many against the classes (a vocabulary shard: 65536 rows x 19008 classes) the walk goes over
+// blocks of ROWS instead, each with the whole vocabulary: dE of a block is then complete after its one launch (written
+// once, no compensation buffer of [b, d]) and it is dC that is carried from block to block, as a pair of 16-bit
+// numbers with a [v, d] compensation buffer.  Same kernels, the roles of the two outputs exchanged.
 // Both products run on the tile loop of cce_tile4.h (direct-to-LDS loads, LDS transpose reads for the
 // operand whose reduction index is the row index).  Everything is enqueued on the caller's stream; nothing
 // is allocated, no host synchronisation.
@@ -37,11 +41,14 @@ struct ProductParams {
   uint16_t* de_hi;      // dE accumulated as a pair of 16-bit values hi + lo: hi is the caller's d_e in the input type
   uint16_t* de_lo;      //   (rows of e), lo the compensation term in the workspace ([b][d], rows by valid-row number)
   int64_t ld_de;        // row stride of d_e (elements)
-  int first_chunk;      // nothing accumulated yet: the pair is written, not read
+  int first_chunk;      // nothing accumulated yet: the pair is written, not read (de_lo == nullptr: the 16-bit d_e is
+                        //   complete with this launch and written alone)
   void* d_c;            // first class of the chunk
   int64_t ld_dc;        // row stride of d_c (elements)
   int dc_fp32;
   int dc_accumulate;    // d_c (fp32) is added to, not written
+  uint16_t* dc_lo;      // a 16-bit d_c carried over blocks of rows as a pair hi + lo: hi is d_c, lo this [n_cls][d]
+  int dc_first;         //   compensation term in the workspace (nullptr: d_c is written once); the first block writes the pair
   int de_rows_by_number;  // the fp32 d_e is indexed by valid-row number (a [b, d] accumulator), not by row of e
   int64_t b;
   int d;
@@ -130,7 +137,7 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
       const uint4* src = reinterpret_cast<const uint4*>(p.de_f32 + o.re * p.ld_de + cg);
       o.a = src[0];
       o.b = src[1];
-    } else if (!p.first_chunk) {
+    } else if (!p.first_chunk) {  // (never with de_lo == nullptr: a d_e written alone is a first chunk)
       o.a = *reinterpret_cast<const uint4*>(p.de_hi + o.re * p.ld_de + cg);
       o.b = *reinterpret_cast<const uint4*>(p.de_lo + ri * p.d + cg);
     }
@@ -177,7 +184,7 @@ __device__ __forceinline__ void dense_de_tile(const ProductParams& p, int tm, in
         lo_out[k] = Elem<T>::pack2(rest[0], rest[1]);
       }
       *hi_ptr = make_uint4(ho[0], ho[1], ho[2], ho[3]);
-      *lo_ptr = make_uint4(lo_out[0], lo_out[1], lo_out[2], lo_out[3]);
+      if (p.de_lo != nullptr) *lo_ptr = make_uint4(lo_out[0], lo_out[1], lo_out[2], lo_out[3]);
     }
   });
 }
@@ -209,6 +216,54 @@ __device__ __forceinline__ void dense_dc_tile(const ProductParams& p, int tm, in
   Tile::prefetch(s, loop, ptrs, ids, g);
   Tile::run(acc, s, loop, ptrs, ids, smem, g);
 
+  if (p.dc_lo != nullptr) {
+    // a 16-bit dC carried over blocks of rows: value so far = hi + lo, as dE is carried over chunks of classes
+    struct Old {
+      int ok;
+      uint4 a, b;
+    };
+    auto fetch = [&](int row, int col) {
+      Old o;
+      o.ok = 0;
+      o.a = make_uint4(0u, 0u, 0u, 0u);
+      o.b = make_uint4(0u, 0u, 0u, 0u);
+      const int cls = m0 + row;
+      const int cg = n0 + col;
+      if (cls >= p.n_cls || cg >= p.d) return o;
+      o.ok = 1;
+      if (!p.dc_first) {
+        o.a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(p.d_c) + static_cast<int64_t>(cls) * p.ld_dc + cg);
+        o.b = *reinterpret_cast<const uint4*>(p.dc_lo + static_cast<int64_t>(cls) * p.d + cg);
+      }
+      return o;
+    };
+    typename Tile::template Rmw<Old> rmw;
+    Tile::rmw_begin(rmw, g, fetch);
+    Tile::for_each_row_piece_rmw(acc, smem, g, rmw, fetch, [&](int row, int col, const float (&v)[8], const Old& o) {
+      if (!o.ok) return;
+      const int cls = m0 + row;
+      const int cg = n0 + col;
+      uint4* hi_ptr = reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.d_c) + static_cast<int64_t>(cls) * p.ld_dc + cg);
+      uint4* lo_ptr = reinterpret_cast<uint4*>(p.dc_lo + static_cast<int64_t>(cls) * p.d + cg);
+      const uint32_t hw[4] = {o.a.x, o.a.y, o.a.z, o.a.w}, lw[4] = {o.b.x, o.b.y, o.b.z, o.b.w};
+      uint32_t ho[4], lo_out[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float t[2], rest[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          t[h] = (Elem<T>::to_float(static_cast<uint16_t>(hw[k] >> (16 * h))) +
+                  Elem<T>::to_float(static_cast<uint16_t>(lw[k] >> (16 * h)))) + v[2 * k + h];
+        ho[k] = Elem<T>::pack2(t[0], t[1]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) rest[h] = t[h] - Elem<T>::to_float(static_cast<uint16_t>(ho[k] >> (16 * h)));
+        lo_out[k] = Elem<T>::pack2(rest[0], rest[1]);
+      }
+      *hi_ptr = make_uint4(ho[0], ho[1], ho[2], ho[3]);
+      *lo_ptr = make_uint4(lo_out[0], lo_out[1], lo_out[2], lo_out[3]);
+    });
+    return;
+  }
   Tile::for_each_row_piece(acc, smem, g, [&](int row, int col, const float (&v)[8]) {
     const int cls = m0 + row;
     const int cg = n0 + col;
@@ -368,6 +423,48 @@ static int64_t dense_chunk_classes_uncached(int64_t b, int64_t v, int64_t d, int
 
 static int64_t align256(int64_t x) { return (x + 255) / 256 * 256; }
 
+// How cce_backward_dense walks the [b, v] plane for a dz buffer of at most `max_dz_bytes`.
+//   by classes  chunks of `unit` classes, all b rows each: dC of a chunk is complete, dE is carried over the chunks
+//               (a 16-bit dE as a pair: fixed part of the workspace = its [b, d] compensation term);
+//   by rows     blocks of `unit` rows, all v classes each: dE of a block is complete, dC is carried over the blocks
+//               (fixed part = a [v, d] compensation term).
+// Both walks take the same number of launches for the same buffer; what is carried is read and written once per
+// launch, and its compensation term sits in the workspace for the whole call, so the walk goes by rows where the
+// rows outnumber the classes two to one (measured, E [65536, 3584] x C [19008, 3584]: 36.1 ms and 581 MB by classes
+// with 1024-class chunks, against the same 130 MB of dz by rows).  Only with 16-bit gradients: an fp32 dE is its own
+// accumulator.  unit == 0: not even the smallest plan (256 classes / rows) fits.
+struct DensePlan {
+  bool by_rows;
+  int64_t unit;
+  int64_t fixed_bytes;
+  int64_t dz_bytes;
+};
+static bool dense_walks_by_rows(int64_t b, int64_t v, bool gradients_16bit) {
+  return gradients_16bit && b >= 2 * ((v + 255) / 256 * 256);
+}
+static DensePlan dense_plan(int64_t b, int64_t v, int64_t d, bool gradients_16bit, int64_t max_dz_bytes) {
+  DensePlan pl;
+  pl.by_rows = dense_walks_by_rows(b, v, gradients_16bit);
+  if (pl.by_rows) {
+    const int64_t v_pad = (v + 255) / 256 * 256;
+    const int64_t b_pad = (b + 255) / 256 * 256;
+    pl.fixed_bytes = align256(v * d * 2);
+    int64_t rb = max_dz_bytes / (v_pad * 2) / 256 * 256;
+    if (rb > b_pad) rb = b_pad;
+    if (rb >= 256) {  // blocks of equal size: the last one is not a sliver
+      const int64_t blocks = (b + rb - 1) / rb;
+      rb = ((b + blocks - 1) / blocks + 255) / 256 * 256;
+    }
+    pl.unit = rb >= 256 ? rb : 0;
+    pl.dz_bytes = align256(pl.unit * v_pad * 2);
+  } else {
+    pl.fixed_bytes = gradients_16bit ? align256(b * d * 2) : 0;
+    pl.unit = dense_chunk_classes(b, v, d, max_dz_bytes, true, true);
+    pl.dz_bytes = align256(b * pl.unit * 2);
+  }
+  return pl;
+}
+
 }  // namespace cce
 
 using namespace cce;
@@ -375,10 +472,26 @@ using namespace cce;
 extern "C" int64_t cce_backward_dense_workspace_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace,
                                                       int64_t max_dz_bytes) {
   if (b <= 0 || v <= 0 || d <= 0) return 0;
-  int64_t vc = dense_chunk_classes(b, v, d, max_dz_bytes, true, true);
-  if (vc == 0) vc = 256;  // the smallest plan
-  const int64_t comp = d_e_in_workspace ? align256(b * d * 2) : 0;  // the compensation half of dE
-  return comp + align256(b * vc * 2);
+  DensePlan pl = dense_plan(b, v, d, d_e_in_workspace != 0, max_dz_bytes);
+  if (pl.unit == 0) {  // the smallest plan
+    const int64_t v_pad = (v + 255) / 256 * 256;
+    pl.dz_bytes = align256(256 * (pl.by_rows ? v_pad : b) * 2);
+  }
+  return pl.fixed_bytes + pl.dz_bytes;
+}
+
+extern "C" int64_t cce_backward_dense_fixed_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace) {
+  if (b <= 0 || v <= 0 || d <= 0) return 0;
+  return dense_plan(b, v, d, d_e_in_workspace != 0, 0).fixed_bytes;
+}
+
+extern "C" int64_t cce_backward_dense_dz_bytes(int64_t b, int64_t v, int64_t d, int d_e_in_workspace, int64_t units) {
+  if (b <= 0 || v <= 0 || d <= 0 || units <= 0) return 0;
+  const int64_t v_pad = (v + 255) / 256 * 256;
+  const int64_t b_pad = (b + 255) / 256 * 256;
+  const int64_t u = (units + 255) / 256 * 256;
+  if (dense_walks_by_rows(b, v, d_e_in_workspace != 0)) return (u < b_pad ? u : b_pad) * v_pad * 2;
+  return b * (u < v_pad ? u : v_pad) * 2;
 }
 
 extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias,
@@ -408,13 +521,17 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
     return workspace == nullptr ? CCE_ERR_WORKSPACE_TOO_SMALL : CCE_ERR_MISALIGNED;
 
-  // ---- plan: [16-bit compensation term of dE][dz chunk] ----------------------------------------------------
+  // ---- plan: [16-bit compensation term of the gradient that is carried][dz buffer] ------------------------------
   const bool split_de = (d_e != nullptr) && !d_e_is_fp32;
-  const int64_t comp_bytes = split_de ? align256(b * d * 2) : 0;
+  // (the walk by rows needs the caller to have sized the workspace for it: a 16-bit d_e is what the size query's
+  // flag says, and a d_c in fp32 beside it is added to in place)
+  const bool by_rows = dense_walks_by_rows(b, v, split_de);
+  const int64_t comp_bytes = dense_plan(b, v, d, split_de, 0).fixed_bytes;
   // the plan the size query made (both gradients wanted), so that its answer always suffices
-  const int64_t vc = dense_chunk_classes(b, v, d, workspace_bytes - comp_bytes, true, true);
-  if (vc == 0) return CCE_ERR_WORKSPACE_TOO_SMALL;
+  const DensePlan plan = dense_plan(b, v, d, split_de, workspace_bytes - comp_bytes);
+  if (plan.unit == 0) return CCE_ERR_WORKSPACE_TOO_SMALL;
   uint16_t* dz = reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + comp_bytes);
+  const int64_t vc = by_rows ? (v + 255) / 256 * 256 : plan.unit;
   const int64_t ldz = vc;
 
   ProductParams p;
@@ -426,11 +543,13 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   p.valids = valids;
   p.de_f32 = split_de ? nullptr : static_cast<float*>(d_e);
   p.de_hi = split_de ? static_cast<uint16_t*>(d_e) : nullptr;
-  p.de_lo = split_de ? static_cast<uint16_t*>(workspace) : nullptr;
+  p.de_lo = (split_de && !by_rows) ? static_cast<uint16_t*>(workspace) : nullptr;
   p.ld_de = stride_e;
   p.dc_fp32 = d_c_is_fp32;
   p.ld_dc = stride_cv;
   p.dc_accumulate = 0;
+  p.dc_lo = nullptr;
+  p.dc_first = 1;
   p.de_rows_by_number = 0;
   p.b = b;
   p.d = static_cast<int>(d);
@@ -449,6 +568,56 @@ extern "C" int cce_backward_dense(const void* e, const void* c, const void* bias
   } while (0)
 
   const size_t es = 2;
+  if (by_rows) {
+    // ---- blocks of rows, the whole vocabulary each ------------------------------------------------------------
+    const int64_t rb = plan.unit;
+    p.c = static_cast<const uint16_t*>(c);
+    p.n_cls = static_cast<int>(v);
+    p.first_chunk = 1;  // d_e of a block is complete with its launch
+    p.tiles_n = tiles_n;
+    p.d_c = d_c;
+    p.dc_lo = (d_c != nullptr && !d_c_is_fp32) ? static_cast<uint16_t*>(workspace) : nullptr;
+    p.dc_tiles = (d_c != nullptr) ? static_cast<int>((v + 255) / 256) * tiles_n : 0;
+    p.dc_per_xcd = (p.dc_tiles + 7) / 8;
+    for (int64_t r0 = 0; r0 < b; r0 += rb) {
+      const int64_t n = (b - r0 < rb) ? (b - r0) : rb;
+      // Rows are numbered through valids when there is one (absolute rows of e: only the list moves on); without
+      // one the block is the rows [r0, r0 + n) of e, and everything indexed by row moves with it.
+      const int64_t shift_rows = (valids == nullptr) ? r0 : 0;
+      const unsigned char* e_blk = static_cast<const unsigned char*>(e) + shift_rows * stride_e * es;
+      const int32_t* valids_blk = valids ? valids + r0 : nullptr;
+      const float* d_out_blk = d_out_is_scalar ? d_out : d_out + shift_rows;
+      const float* d_lse_blk = d_lse ? d_lse + shift_rows : nullptr;
+      int st = dense_dz_launch(e_blk, c, bias, lse + r0, d_out_blk, d_out_is_scalar, d_lse_blk, valids_blk,
+                               targets + shift_rows, dz, ldz, 0, 1, n_rows - shift_rows, n, v, d, stride_e, stride_cv,
+                               stride_cd, grad_scale, shift, target_offset, softcap, dtype, stream);
+      if (st != CCE_OK) return st;
+      p.e = reinterpret_cast<const uint16_t*>(e_blk);
+      p.valids = valids_blk;
+      p.de_hi = static_cast<uint16_t*>(d_e) + shift_rows * stride_e;
+      p.b = n;
+      p.dc_first = (r0 == 0) ? 1 : 0;
+      p.dc_accumulate = (r0 == 0) ? 0 : 1;  // an fp32 d_c is written by the first block and added to by the others
+      p.de_tiles = static_cast<int>((n + 255) / 256) * tiles_n;
+      p.de_per_xcd = (p.de_tiles + 7) / 8;
+      p.de_first = (v > n) ? 1 : 0;
+      const int blocks = (p.dc_per_xcd + p.de_per_xcd) * 8;
+      if (dtype == CCE_DTYPE_BF16) CCE_LAUNCH_PRODUCT((dense_products_kernel<BF16, true>), blocks);
+      else CCE_LAUNCH_PRODUCT((dense_products_kernel<F16, true>), blocks);
+      if (d_bias != nullptr) {
+        const unsigned cblocks = static_cast<unsigned>((v + 63) / 64);
+        if (dtype == CCE_DTYPE_BF16)
+          hipLaunchKernelGGL(dz_colsum_kernel<BF16>, dim3(cblocks), dim3(1024), 0, stream, dz, ldz, n, static_cast<int>(v),
+                             d_bias);
+        else
+          hipLaunchKernelGGL(dz_colsum_kernel<F16>, dim3(cblocks), dim3(1024), 0, stream, dz, ldz, n, static_cast<int>(v),
+                             d_bias);
+      }
+      err = hipGetLastError();
+      if (err != hipSuccess) return status_from_hip(err);
+    }
+    return status_from_hip(hipGetLastError());
+  }
   for (int64_t v0 = 0; v0 < v; v0 += vc) {
     const int64_t n = (v - v0 < vc) ? (v - v0) : vc;
     const unsigned char* c_chunk = static_cast<const unsigned char*>(c) + v0 * stride_cv * es;
@@ -536,6 +705,8 @@ extern "C" int cce_backward_products(const void* dz, int64_t ldz, const void* c,
   p.ld_dc = ld_dc;
   p.dc_fp32 = 1;
   p.dc_accumulate = d_c_accumulate;
+  p.dc_lo = nullptr;
+  p.dc_first = 1;
   p.b = b;
   p.d = static_cast<int>(d);
   p.n_cls = static_cast<int>(n_cls);

@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "li
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1}
 STAT_ROWS = 32
 STAT_COLS = 32
@@ -54,6 +54,8 @@ _SIGNATURES = {
     ),
     "cce_count_flagged_cells": (_i32, [_ptr, _ptr, _i64, _i64, _f32, _ptr, _ptr]),
     "cce_backward_dense_workspace_bytes": (_i64, [_i64, _i64, _i64, _i32, _i64]),
+    "cce_backward_dense_fixed_bytes": (_i64, [_i64, _i64, _i64, _i32]),
+    "cce_backward_dense_dz_bytes": (_i64, [_i64, _i64, _i64, _i32, _i64]),
     "cce_backward_dense": (
         _i32,
         [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64]

@@ -20,15 +20,18 @@ from cut_cross_entropy.utils import TensorInfo
 # compensation buffer (dE is summed over the chunks as a pair of 16-bit numbers).
 DENSE_DZ_BYTES = 256 << 20
 
-# ... but never so small that a chunk holds fewer classes than this: with many rows (B = 65536: 2048 classes in
-# 256 MB) the tiles of dE have a short reduction, their fetch and read-modify-write of dE weigh as much as their
-# products, and dE is passed over once per chunk (measured, backward of E [65536, 3584] x C [19008, 3584]: 24.9 ms
-# with 256 MB, 21.7 with 512, 21.1 with 1024).  The buffer then grows with B like E and dE themselves do.
+# ... but never so small that a chunk holds fewer classes than this (a block fewer rows, where the library walks by
+# blocks of rows: 16-bit gradients and at least twice as many rows as classes): the tiles of the gradient that is
+# carried between the launches then have a short reduction, their fetch and read-modify-write weigh as much as their
+# products, and that gradient is passed over once per launch.  The buffer then grows with the problem like its
+# operands do (E [32768, 4096] x C [128256, 4096], by classes: 256 MB hold 4096 classes; E [65536, 3584] x
+# C [19008, 3584], by rows: 256 MB hold 6912 rows, 22.6 ms, against 27.9 ms with 55 MB).
 DENSE_DZ_MIN_CLASSES = 4096
 
 
-def _dz_budget(B: int) -> int:
-    return max(int(DENSE_DZ_BYTES), 2 * int(B) * int(DENSE_DZ_MIN_CLASSES))
+def _dz_budget(lib, B: int, V: int, D: int, de_16bit: bool) -> int:
+    return max(int(DENSE_DZ_BYTES),
+               lib.cce_backward_dense_dz_bytes(B, V, D, 1 if de_16bit else 0, int(DENSE_DZ_MIN_CLASSES)))
 
 # With the gradient filter on, the ownership kernels pay per surviving sub-tile and the dense path pays for
 # the whole plane once.  Measured on MI355X the two cross where 0.177 of the 32 x 32 cells of the forward
@@ -50,7 +53,8 @@ DENSE_WHEN_FLAGGED_ABOVE = 0.17
 FILTERED_BACKWARD_PATH = "auto"
 # A filtered backward that changes to the unfiltered path BY ITSELF may take at most
 #     max(DENSE_WORKSPACE_LIMIT_BYTES, DENSE_WORKSPACE_LIMIT_OPERANDS x (bytes of E + bytes of C))
-# of workspace (the dz chunk, plus the [B, D] 16-bit compensation buffer of dE): the ownership kernels need well
+# of workspace (the dz buffer, plus the 16-bit compensation buffer of the gradient that is carried between launches:
+# [B, D] for dE, or [V, D] for dC where rows outnumber classes two to one): the ownership kernels need well
 # under 16 MB, and a caller who picked a filtered preset did not ask for more.  The defaults, 256 MB and 1.0, say:
 # never more than the operands the caller already holds take themselves, and 256 MB where they are smaller (the
 # second term matters when rows are many: at E [65536, 3584] x C [19008, 3584] the compensation buffer alone is
@@ -109,17 +113,19 @@ def reset_backward_path_memory() -> None:
 def _auto_dense_dz_budget(lib, B: int, V: int, D: int, de_16bit: bool, operand_bytes: int) -> Optional[int]:
     """dz chunk bytes a filtered backward may use when it changes to the unfiltered path by itself, or None when
     the workspace limit leaves no room for chunks of a useful size."""
-    budget = _dz_budget(B)
+    budget = _dz_budget(lib, B, V, D, de_16bit)
     if DENSE_WORKSPACE_LIMIT_BYTES is None:
         return budget
     limit = max(int(DENSE_WORKSPACE_LIMIT_BYTES), int(DENSE_WORKSPACE_LIMIT_OPERANDS * operand_bytes))
-    comp = lib.cce_backward_dense_workspace_bytes(B, V, D, 1 if de_16bit else 0, 0) - \
-        lib.cce_backward_dense_workspace_bytes(B, V, D, 0, 0)
-    # Chunks of fewer than AUTO_DENSE_MIN_CLASSES classes are not worth having: every chunk passes over all of dE, and
-    # its products reduce over a handful of stages (measured, backward of E [15356, 4096] x C [128256, 4096]: 226 ms
-    # with 256 classes per chunk, 45 ms with 2048, 39 ms with 8192, against 168 ms on the ownership kernels).
-    room = limit - comp
-    if room < 2 * B * min(AUTO_DENSE_MIN_CLASSES, (V + 255) // 256 * 256):
+    # what the unfiltered backward keeps for the whole call (the compensation term of the gradient it carries from
+    # launch to launch: [B, D], or [V, D] where it walks by blocks of rows)
+    fixed = lib.cce_backward_dense_fixed_bytes(B, V, D, 1 if de_16bit else 0)
+    # dz buffers of fewer than AUTO_DENSE_MIN_CLASSES classes per chunk (rows per block) are not worth having: every
+    # launch passes over all of the carried gradient, and its products reduce over a handful of stages (measured,
+    # backward of E [15356, 4096] x C [128256, 4096]: 226 ms with 256 classes per chunk, 45 ms with 2048, 39 ms with
+    # 8192, against 168 ms on the ownership kernels).
+    room = limit - fixed
+    if room < lib.cce_backward_dense_dz_bytes(B, V, D, 1 if de_16bit else 0, int(AUTO_DENSE_MIN_CLASSES)):
         return None
     return min(budget, room)
 
@@ -274,7 +280,7 @@ def cce_backward_kernel(
     layout_ok = _dense_layout_ok(e, c)
     de_dense = want_de and layout_ok and not e_filtered
     dc_dense = (want_dc or want_dbias) and layout_ok and not c_filtered
-    dz_budget = _dz_budget(n_valid_rows)
+    dz_budget = _dz_budget(lib, n_valid_rows, c.size(0), e.size(1), de_dense and e_info.dtype != torch.float32)
     some_filtered = (want_de and not de_dense) or ((want_dc or want_dbias) and not dc_dense)
     if (some_filtered and layout_ok and tile_max is not None and filter_eps is not None and filter_eps > 0
             and lse.numel() > 0):

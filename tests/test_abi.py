@@ -30,7 +30,8 @@ def test_header_declares_the_expected_entry_points():
     for want in ("cce_version", "cce_error_string", "cce_tile_stat_elems", "cce_lse_forward_workspace_bytes",
                  "cce_lse_forward", "cce_indexed_neg_dot", "cce_backward_workspace_bytes", "cce_backward",
                  "cce_backward_dz", "cce_lse_forward_static", "cce_lse_forward_static_init", "cce_backward_dense",
-                 "cce_backward_dense_workspace_bytes", "cce_count_flagged_cells", "cce_backward_products"):
+                 "cce_backward_dense_workspace_bytes", "cce_backward_dense_fixed_bytes", "cce_backward_dense_dz_bytes",
+                 "cce_count_flagged_cells", "cce_backward_products"):
         assert want in names
 
 
@@ -77,3 +78,28 @@ def test_header_constants_match_binding():
     assert int(re.search(r"#define CCE_DTYPE_F16 (\d+)", text).group(1)) == 1
     m = re.search(r"#define CCE_STATIC_SCRATCH_BYTES \((\d+) \* (\d+) \* (\d+)\)", text)
     assert int(m.group(1)) * int(m.group(2)) * int(m.group(3)) == _hip.STATIC_SCRATCH_BYTES
+
+
+def test_dense_backward_plans_by_classes_or_by_rows():
+    """Host-only size queries of the unfiltered backward: with 16-bit gradients and at least twice as many rows as
+    classes the walk goes by blocks of rows and the compensation term in the workspace is [v, d], else [b, d]."""
+    lib = _lib()
+    a256 = lambda x: (x + 255) // 256 * 256
+    # rows few against classes: by classes; fixed part = compensation term of dE
+    assert lib.cce_backward_dense_fixed_bytes(8192, 256000, 2304, 1) == a256(8192 * 2304 * 2)
+    assert lib.cce_backward_dense_fixed_bytes(8192, 256000, 2304, 0) == 0
+    assert lib.cce_backward_dense_dz_bytes(8192, 256000, 2304, 1, 1024) == 8192 * 1024 * 2
+    # a vocabulary shard: by rows; fixed part = compensation term of dC; a dz unit is 256 rows of all classes
+    B, V, D = 65536, 19008, 3584
+    v_pad = a256(V)
+    assert lib.cce_backward_dense_fixed_bytes(B, V, D, 1) == a256(V * D * 2)
+    assert lib.cce_backward_dense_fixed_bytes(B, V, D, 0) == 0           # fp32 gradients: by classes, nothing fixed
+    assert lib.cce_backward_dense_dz_bytes(B, V, D, 1, 1024) == 1024 * v_pad * 2
+    assert lib.cce_backward_dense_dz_bytes(B, V, D, 0, 1024) == B * 1024 * 2
+    # the whole workspace: fixed part + a dz buffer inside the budget, never below one 256-row block
+    for budget in (0, 64 << 20, 256 << 20, 1 << 32):
+        total = lib.cce_backward_dense_workspace_bytes(B, V, D, 1, budget)
+        dz = total - a256(V * D * 2)
+        assert dz % (256 * v_pad * 2) == 0 and dz >= 256 * v_pad * 2
+        assert dz <= max(budget, 256 * v_pad * 2)
+        assert dz <= a256(B) * v_pad * 2

@@ -43,11 +43,15 @@ def test_workloads_name_the_configurations_of_the_baseline():
 
 
 class _FakeLib:
-    """cce_backward_dense_workspace_bytes of the library, restated: the dz chunk plus, for a 16-bit dE, [B, D] x 2."""
+    """The two size queries of the library the rule uses, restated for the walk by classes."""
 
     @staticmethod
-    def cce_backward_dense_workspace_bytes(b, v, d, de_16bit, max_dz_bytes):
-        return (2 * b * d if de_16bit else 0) + 12345  # the dz part cancels in the difference the host takes
+    def cce_backward_dense_fixed_bytes(b, v, d, de_16bit):
+        return 2 * b * d if de_16bit else 0
+
+    @staticmethod
+    def cce_backward_dense_dz_bytes(b, v, d, de_16bit, units):
+        return 2 * b * min((units + 255) // 256 * 256, (v + 255) // 256 * 256)
 
 
 @pytest.mark.parametrize(
@@ -59,7 +63,8 @@ class _FakeLib:
         (15356, 128256, 4096, 192 << 20, 0.0, "room"),
         # the operand rule: E + C = 1122 MB, so the 256 MB floor does not bind and the budget is DENSE_DZ_BYTES
         (15356, 128256, 4096, 256 << 20, 1.0, "budget"),
-        # c5-shard-like: the compensation buffer alone (448 MB) exceeds 256 MB; operands (578 MB) leave 130 MB >= 128 MB
+        # many rows, walked by classes: the compensation buffer alone (448 MB) exceeds 256 MB; the operands (578 MB)
+        # leave 130 MB >= 128 MB
         (65536, 19008, 3584, 256 << 20, 0.0, None),
         (65536, 19008, 3584, 256 << 20, 1.0, "room"),
         # a vocabulary smaller than 1024 classes needs room for itself only
@@ -79,9 +84,9 @@ def test_workspace_rule_of_the_self_chosen_unfiltered_backward(monkeypatch, B, V
     if expect is None:
         assert got is None
     elif expect == "room":
-        assert got == room and got < bw._dz_budget(B)
+        assert got == room and got < bw._dz_budget(_FakeLib, B, V, D, True)
         assert got >= 2 * B * min(bw.AUTO_DENSE_MIN_CLASSES, (V + 255) // 256 * 256)
     else:
-        assert got == bw._dz_budget(B) and got <= room
+        assert got == bw._dz_budget(_FakeLib, B, V, D, True) and got <= room
     monkeypatch.setattr(bw, "DENSE_WORKSPACE_LIMIT_BYTES", None)
-    assert bw._auto_dense_dz_budget(_FakeLib, B, V, D, True, operand_bytes) == bw._dz_budget(B)
+    assert bw._auto_dense_dz_budget(_FakeLib, B, V, D, True, operand_bytes) == bw._dz_budget(_FakeLib, B, V, D, True)

@@ -227,11 +227,15 @@ def test_backward_dz_abi(dtype, softcap, has_bias, with_dlse, shape):
 @pytest.mark.parametrize("has_bias", [False, True])
 @pytest.mark.parametrize("fp32_out", [False, True])
 @pytest.mark.parametrize("shape,dz_budget", [((256, 512, 128), 0), ((255, 507, 64), 0), ((700, 1300, 192), 0),
-                                             ((300, 1100, 320), 1 << 30), ((520, 2100, 576), 520 * 768 * 2)])
+                                             ((300, 1100, 320), 1 << 30), ((520, 2100, 576), 520 * 768 * 2),
+                                             ((1500, 300, 128), 0), ((1500, 300, 128), 1 << 30),
+                                             ((2100, 500, 320), 768 * 512 * 2), ((900, 130, 64), 0)])
 def test_backward_dense_abi(dtype, softcap, has_bias, fp32_out, shape, dz_budget):
     """cce_backward_dense (dz chunks + hand-written dE / dC products, one call) vs the closed-form dense
     gradients: several chunks (smallest workspace), one chunk (large workspace), ragged rows, classes and
-    columns, rows gathered through valids, upstream d_lse."""
+    columns, rows gathered through valids, upstream d_lse.  The last four shapes have more than twice as many
+    valid rows as classes: with 16-bit gradients the walk then goes by blocks of rows (five blocks of 256, one
+    block, three blocks of 768 less a remainder, three of 256), dC carried between them as a 16-bit pair."""
     from oracle import dense_lce
 
     lib = _lib()

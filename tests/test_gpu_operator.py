@@ -214,6 +214,53 @@ def test_unfiltered_backward_takes_the_dense_path(monkeypatch, impl, with_valids
     assert len(calls) == 2
 
 
+@pytest.mark.parametrize("with_valids", [False, True])
+@pytest.mark.parametrize("reduction", ["mean", "none"])
+def test_unfiltered_backward_walks_by_rows_where_rows_outnumber_classes(monkeypatch, with_valids, reduction):
+    """A vocabulary shard in miniature: five times as many rows as classes.  The unfiltered backward then walks blocks
+    of rows with the whole vocabulary each (dE complete per block, dC carried between the blocks as a 16-bit pair); a
+    small dz budget makes it several blocks.  Rows indexed directly and through valids (shift, ignored labels), a
+    scalar and a per-row upstream gradient."""
+    from cut_cross_entropy import _hip
+    from cut_cross_entropy import cce_backward as bw
+    from cut_cross_entropy import linear_cross_entropy
+    from oracle import dense_lce
+
+    N, V, D = 1536, 300, 128
+    lib = _hip.load()
+    assert lib.cce_backward_dense_fixed_bytes(N, V, D, 1) == (V * D * 2 + 255) // 256 * 256  # by rows: the term of dC
+    monkeypatch.setattr(bw, "DENSE_DZ_BYTES", 512 * 512 * 2)  # 512 rows x 512 (padded) classes: three blocks
+    monkeypatch.setattr(bw, "DENSE_DZ_MIN_CLASSES", 0)
+    e, c, t, _ = make_inputs(N, V, D, torch.bfloat16, seed=5, invalid_frac=0.1 if with_valids else 0.0)
+    shift = 1 if with_valids else 0
+    g = torch.Generator().manual_seed(3)
+    w = torch.rand((N - shift,), generator=g) + 0.5  # reduction "none" returns one loss per row that has a target
+    ed, cd = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    e64, c64 = e.double().requires_grad_(True), c.double().requires_grad_(True)
+    for numel in (e.numel(), c.numel()):  # blocks full of NaN for the allocator to hand out
+        torch.full((numel,), float("nan"), dtype=torch.bfloat16, device="cuda")
+    loss = linear_cross_entropy(ed, cd, t.cuda(), softcap=25.0, impl="cce_exact", shift=shift, reduction=reduction)
+    want, _ = dense_lce.dense_linear_cross_entropy(e64, c64, t, softcap=25.0, shift=shift, reduction=reduction)
+    if reduction == "none":
+        loss = (loss * w.cuda()).sum() / N
+        want = (want * w.double()).sum() / N
+    loss.backward()
+    want.backward()
+    assert abs(loss.item() - want.item()) <= 1e-3 * abs(want.item())
+    scale = 1.0 / N
+    assert torch.allclose(ed.grad.double().cpu(), e64.grad, atol=2e-2 * scale, rtol=2e-2)
+    assert torch.allclose(cd.grad.double().cpu(), c64.grad, atol=2e-2 * scale, rtol=2e-2)
+    # one block (the default budget) gives the same dC up to the rounding of the 16-bit pair
+    monkeypatch.setattr(bw, "DENSE_DZ_BYTES", 256 << 20)
+    ed2, cd2 = e.cuda().requires_grad_(True), c.cuda().requires_grad_(True)
+    loss2 = linear_cross_entropy(ed2, cd2, t.cuda(), softcap=25.0, impl="cce_exact", shift=shift, reduction=reduction)
+    if reduction == "none":
+        loss2 = (loss2 * w.cuda()).sum() / N
+    loss2.backward()
+    assert torch.equal(ed2.grad, ed.grad)  # dE of a row does not depend on how the rows are cut into blocks
+    assert torch.allclose(cd2.grad.float(), cd.grad.float(), atol=1e-2 * scale, rtol=1e-2)
+
+
 def test_filtered_backward_runs_dense_when_most_cells_can_survive(monkeypatch):
     """Near-uniform soft-max over few classes: every cell's bound exp(max logit - min lse) is above
     filter_eps, so the backward runs unfiltered (and is then exact) -- from the FIRST step on: the first backward
