@@ -1190,9 +1190,18 @@ __global__ __launch_bounds__(kBwdThreads, LIGHT ? 2 : 1) void bwd_owner_fast_ker
   mfma_drain_all();  // the last product MFMAs, before anything else reads the accumulators
   const bool out_fp32 = IS_DE ? (p.de_fp32 != 0) : (p.dc_fp32 != 0);
   if constexpr (LIGHT) {
-    if (write_out && !touched) {  // nothing survived for this class group: its rows are zeros
-#pragma unroll 1
-      for (int ci = 0; ci < nchunks; ++ci) store_chunk_direct(ci, acc[0]);
+    if (write_out && !touched) {
+      // Nothing survived for this class group: its rows are zeros, written as whole 16-byte pieces, a wave
+      // instruction inside one row (the launcher guarantees 16-byte aligned rows and D a multiple of 128).
+      const int ppr = (d_end - d_begin) / 8;  // 16-byte pieces per row
+      const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+      for (int j = tid; j < 32 * ppr; j += kBwdThreads) {
+        const int row = j / ppr;
+        const int id = own_ids[row];
+        if (id >= 0)
+          *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p.d_c) + static_cast<int64_t>(id) * own_sr + d_begin +
+                                    (j - row * ppr) * 8) = zero;
+      }
     }
   } else if (write_out && (touched || !IS_DE)) {  // dC rows are always written; the launcher guarantees 16-byte aligned rows
     // The accumulators hold the tile transposed (lane = own row, registers = columns): stored as they
