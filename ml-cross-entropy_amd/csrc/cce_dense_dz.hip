@@ -301,7 +301,12 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz16_kernel(DzParams p) {
     Fast::set_class_tile(src, reinterpret_cast<const unsigned char*>(p.c) + v0 * p.stride_cv * 2, left, wave);
   };
 
-  // What the rows of this workgroup need, fixed for the whole item (published by the first barrier of the main loop).
+  unsigned char* stage = s_stage + wave * kDz16StageBytes;
+  int buf = 0;
+  set_class_tile(vt_begin);
+  Fast::prefetch(src, smem);
+  // What the rows of this workgroup need, fixed for the whole item (published by the first barrier of the main loop;
+  // fetched behind the first stages of the ring, so that the two latencies overlap).
   if (tid < kDzTile) {
     const int64_t i = t0 + tid;
     DzRow r = {INFINITY, 0.0f, 0.0f, -1};
@@ -318,11 +323,6 @@ __global__ __launch_bounds__(kDzThreads, 1) void dense_dz16_kernel(DzParams p) {
     }
     s_rows[tid] = r;
   }
-
-  unsigned char* stage = s_stage + wave * kDz16StageBytes;
-  int buf = 0;
-  set_class_tile(vt_begin);
-  Fast::prefetch(src, smem);
 
   for (int vt = vt_begin; vt < vt_end; ++vt) {
     const int64_t v0 = static_cast<int64_t>(vt) * kDzTile;
