@@ -281,6 +281,39 @@ def test_backward_dense_abi(dtype, softcap, has_bias, fp32_out, shape, dz_budget
     assert (de.cpu()[ignored] == 0).all()
 
 
+@pytest.mark.parametrize("dz_budget", [0, 1 << 30])
+def test_backward_dense_walks_by_rows_with_an_fp32_dc(dz_budget):
+    """More than twice as many rows as classes, a 16-bit d_e and an fp32 d_c: the walk goes by blocks of rows, d_e of a
+    block is written once, and the fp32 d_c is written by the first block and added to in place by the others (no
+    compensation term is used for it).  Rows taken directly (no valids), a scalar upstream gradient."""
+    from oracle import dense_lce
+
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D, dtype = 1300, 200, 192, torch.bfloat16
+    e, c, t, _ = make_inputs(N, V, D, dtype, seed=11)
+    lse = dense_lce.dense_lse(e, c, None, None, torch.float64)
+    d_out = torch.full((N,), 1.0 / N)
+    gt = dense_lce.dense_grads(e, c, t, None, d_out, None, None, None, 0, torch.float64)
+    ed, cd, td = e.to(dev), c.to(dev), t.to(dev)
+    lsed = lse.float().to(dev)
+    do = torch.full((1,), 1.0 / N, device=dev)
+    de = torch.full((N, D), float("nan"), dtype=dtype, device=dev)          # written whole
+    dc = torch.full((V, D), float("nan"), dtype=torch.float32, device=dev)  # written by the first block
+    assert lib.cce_backward_dense_fixed_bytes(N, V, D, 1) == (V * D * 2 + 255) // 256 * 256  # the walk by rows
+    ws_bytes = lib.cce_backward_dense_workspace_bytes(N, V, D, 1, dz_budget)
+    ws = torch.empty((ws_bytes + 256,), dtype=torch.uint8, device=dev)
+    st = lib.cce_backward_dense(
+        ed.data_ptr(), cd.data_ptr(), None, lsed.data_ptr(), do.data_ptr(), 1, None, None, td.data_ptr(),
+        de.data_ptr(), dc.data_ptr(), None, (ws.data_ptr() + 255) // 256 * 256, ws_bytes,
+        N, N, V, D, D, D, 1, 1.0, 0, 1, 0, 0, 0.0, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    assert torch.isfinite(de).all() and torch.isfinite(dc).all()
+    assert torch.allclose(de.cpu().double(), gt[0], atol=2e-2 / N, rtol=2e-2)
+    assert torch.allclose(dc.cpu().double(), gt[1], atol=2e-2 / N, rtol=2e-2)
+
+
 def test_backward_dense_ignores_non_finite_values_it_must_not_read():
     """Rows of e that are not valid and the reduction tails of the product tiles must not leak into the
     gradients: an ignored row full of inf / nan (and such a row as row 0, where absent rows used to point)
