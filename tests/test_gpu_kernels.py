@@ -65,6 +65,48 @@ def test_lse_forward_abi(dtype, softcap, has_bias, shape):
     assert (got >= want - 0.05).all() and (got <= want + 0.05).all()
 
 
+@pytest.mark.parametrize("softcap", [None, 20.0, 50.0])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("shape", [(8192, 20011, 128), (8000, 24576, 192)])
+def test_lse_forward_spans_of_many_tiles(softcap, has_bias, shape):
+    """Thirty-two row blocks leave eight vocabulary spans per row block, each of nine to twelve 256-class tiles: the
+    16x16x32 kernel collects the statistic cells of eight tiles in registers before it stores them, so a span of more
+    than eight tiles has a full batch and a remainder; the ring runs on across the tiles of a span.  Checked against
+    dense fp32 logits formed on the GPU (soft-cap 50 is beyond the fixed-reference range of the epilogue)."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D = shape
+    dtype = torch.bfloat16
+    e, c, _, bias = make_inputs(N, V, D, dtype, seed=3, bias=has_bias)
+    ed, cd = e.to(dev), c.to(dev)
+    bd = bias.to(dev) if bias is not None else None
+    logits = ed.float() @ cd.float().T
+    if bd is not None:
+        logits += bd.float()
+    if softcap is not None:
+        logits = torch.tanh(logits / softcap) * softcap
+    want_lse = torch.logsumexp(logits.double(), dim=1)
+    lse = torch.full((N,), float("nan"), dtype=torch.float32, device=dev)
+    tm = torch.full((lib.cce_tile_stat_elems(N, V),), float("nan"), dtype=torch.float32, device=dev)
+    ws_bytes = lib.cce_lse_forward_workspace_bytes(N, V, D)
+    ws = torch.empty((ws_bytes // 8 + 1,), dtype=torch.int64, device=dev)
+    st = lib.cce_lse_forward(
+        ed.data_ptr(), cd.data_ptr(), bd.data_ptr() if bd is not None else None, None,
+        lse.data_ptr(), None, tm.data_ptr(), ws.data_ptr(), ws.numel() * 8,
+        N, N, V, D, ed.stride(0), cd.stride(0), cd.stride(1),
+        softcap or 0.0, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0, lib.cce_error_string(st)
+    torch.cuda.synchronize()
+    assert torch.allclose(lse.double(), want_lse, atol=2e-4, rtol=2e-5)
+    nr, nc = (N + 31) // 32, (V + 31) // 32
+    pad = torch.full((nr * 32, nc * 32), float("-inf"), device=dev)
+    pad[:N, :V] = logits
+    want = pad.view(nr, 32, nc, 32).amax(dim=(1, 3))
+    got = tm.view(nr, nc)
+    assert torch.isfinite(got).all()
+    assert ((got - want).abs() <= 0.05).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("softcap", [None, 20.0])
 @pytest.mark.parametrize("has_bias", [False, True])
