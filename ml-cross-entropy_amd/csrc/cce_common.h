@@ -150,6 +150,21 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Sum over the 16 lanes of a row (lanes 16 k .. 16 k + 15), left in every lane of the row: four rotations on the
+// vector unit, no LDS crossbar.
+__device__ __forceinline__ float row16_sum(float v) {
+  auto ror = [](float x, auto ctrl) {
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, r);
+  };
+  using std::integral_constant;
+  v += ror(v, integral_constant<int, 0x121>{});  // row_ror:1
+  v += ror(v, integral_constant<int, 0x122>{});  // row_ror:2
+  v += ror(v, integral_constant<int, 0x124>{});  // row_ror:4
+  v += ror(v, integral_constant<int, 0x128>{});  // row_ror:8
+  return v;
+}
+
 // Maximum over the 64 lanes as a wave-uniform value, on the vector unit alone: four rotations inside the rows of 16
 // lanes (after which every lane holds its row's maximum), then lane 15 of rows 0 and 2 broadcast into rows 1 and 3
 // and lane 31 into rows 2 and 3; the last lane then holds the maximum of all.  The shuffles of wave_max() above

@@ -31,6 +31,7 @@ struct LseFwdParams {
   int nrb, nvt, nsplit, nitems, items_per_xcd;
   int stat_cols;
   Softcap sc;
+  float avg_scale;  // ln 2 / b: turns a column sum in log2 units into its share of logit_avg
 };
 
 // 8 waves (two per SIMD, so that one wave's LDS and global traffic issues in the shadow of the
@@ -294,6 +295,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward_kernel(LseFwdParam
 // statistic cells) at a time: 64 soft-capped logits live.
 // ---------------------------------------------------------------------------------------------
 constexpr int kF16WV = 8, kF16WT = 4;  // 16-row blocks per wave: 128 classes x 64 rows
+constexpr int kF16RunBytes = kF16WT * kFwdThreads * static_cast<int>(sizeof(float2));  // running (max, sum) pairs
+constexpr int kF16ColsumBytes = 2 * kFwdTile * static_cast<int>(sizeof(float));       // column sums (logit_avg only)
 static_assert(16 * kF16WV * kFwdNWV == kFwdTile && 16 * kF16WT * kFwdNWT == kFwdTile, "tile is 256 x 256");
 
 // One row block (16 token rows x the wave's 128 classes; 32 values of ONE row per lane) of the epilogue: soft-cap,
@@ -385,6 +388,10 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
   // Eight registers fewer across the main loop, which is what lets the loop and the epilogue go without spills
   // (a reload from scratch memory makes the compiler wait for ALL loads in flight, the ring's included).
   float2* s_run = reinterpret_cast<float2*>(smem + Fast::LDS_BYTES + kFwdBiasBytes) + threadIdx.x;
+  // WANT_LA: the sums of the soft-capped logits of a tile over its 256 rows, per class: [2][256], by tile parity.
+  // The waves add their shares while they are in the epilogue of tile t; the sums leave for memory in the epilogue of
+  // tile t + 1 (or after the last tile): the barriers of the main loop in between order the two.
+  float* s_colsum = reinterpret_cast<float*>(smem + Fast::LDS_BYTES + kFwdBiasBytes + kF16RunBytes);
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -430,6 +437,20 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
   const bool fixed_ref = p.sc.on && p.sc.out_scale < 60.0f;
 #pragma unroll
   for (int ti = 0; ti < kF16WT; ++ti) s_run[ti * kFwdThreads] = make_float2(-INFINITY, 0.0f);
+  if (WANT_LA) s_colsum[tid] = 0.0f;  // 512 threads, 2 x 256 sums; published by the barriers of the first main loop
+  // the sums of the tile that starts at class `first` leave for the running average, and are cleared for the tile after next
+  // (the scale comes as a kernel argument and the address is formed where it is used: a lane constant carried
+  // through the main loop would be parked in scratch memory, and its reload waits for the loads of the ring)
+  auto flush_colsum = [&](int64_t first, int parity) {
+    int t = tid;
+    asm volatile("" : "+v"(t));
+    if (t < kFwdTile) {
+      float* cs = s_colsum + parity * kFwdTile + t;
+      const float sum = *cs;
+      *cs = 0.0f;
+      if (first + t < p.v) unsafeAtomicAdd(p.logit_avg + first + t, sum * p.avg_scale);
+    }
+  };
 
   float stat = 0.0f;  // statistic cells waiting to be written (see the epilogue)
   int buf = 0;
@@ -457,6 +478,14 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
     // ---- epilogue: (bias, mask,) soft-cap, online max / sum-exp ---------------------------------
     const int64_t vw0 = v0 + wv * (16 * kF16WV);  // first class of this wave
     const float* wave_addend = addend + wv * (16 * kF16WV);
+    float la[WANT_LA ? kF16WV : 1][4];  // this lane's sums over its four rows of the tile, log2 units
+    if (WANT_LA) {
+      if (vt > vt_begin) flush_colsum(v0 - kFwdTile, (vt - 1) & 1);
+#pragma unroll
+      for (int vi = 0; vi < kF16WV; ++vi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) la[vi][r] = 0.0f;
+    }
 #pragma unroll
     for (int tp = 0; tp < kF16WT / 2; ++tp) {
       float bm[kF16WV / 2];  // this lane's maxima in the four statistic cells of this row pair
@@ -471,22 +500,11 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
         row_block<GENERAL, WANT_LA>(p.sc, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
         s_run[ti * kFwdThreads] = run;
         if (WANT_LA) {
-          // Column sums over the 16 rows of this block, in natural-log units, added to the running average right away.
-          const float ok = (wrow0 + ti * 16 + r16 < p.b) ? 1.0f : 0.0f;
-          const float inv_b = kLn2 / static_cast<float>(p.b);
-          float* avg = p.logit_avg + vw0 + 4 * kq;  // this lane group's first class of the wave
-          const int left = static_cast<int>(min(p.v - vw0, static_cast<int64_t>(16 * kF16WV))) - 4 * kq;
+          const bool ok = wrow0 + ti * 16 + r16 < p.b;
 #pragma unroll
-          for (int vi = 0; vi < kF16WV; ++vi) {
+          for (int vi = 0; vi < kF16WV; ++vi)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int cls = vi * 16 + r;
-              float cs = (s2[vi][r] == -INFINITY) ? 0.0f : s2[vi][r] * ok;
-#pragma unroll
-              for (int off = 8; off >= 1; off >>= 1) cs += __shfl_xor(cs, off, 64);
-              if (r16 == 0 && cls < left) unsafeAtomicAdd(avg + cls, cs * inv_b);
-            }
-          }
+            for (int r = 0; r < 4; ++r) la[vi][r] += (ok && s2[vi][r] != -INFINITY) ? s2[vi][r] : 0.0f;
         }
       }
 
@@ -503,11 +521,25 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
         }
       }
     }
+    if (WANT_LA) {
+      // Over the 16 lanes that hold the 16 rows of a block (rotations on the vector unit), then one LDS add per class
+      // from the first lane of each group of 16: the four waves that share these classes meet there.
+      float* cs = s_colsum + (vt & 1) * kFwdTile + wv * (16 * kF16WV) + 4 * kq;
+#pragma unroll
+      for (int vi = 0; vi < kF16WV; ++vi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float sum = row16_sum(la[vi][r]);
+          if (r16 == 0) atomicAdd(cs + vi * 16 + r, sum);
+        }
+    }
     if (p.tile_max != nullptr && (((vt - vt_begin) & 7) == 7 || vt + 1 == vt_end)) {
+      int ln = lane;
+      if constexpr (WANT_LA) asm volatile("" : "+v"(ln));  // the cell address is formed here, not carried through the loop
       const int first_vt = vt - ((vt - vt_begin) & 7);
-      const int my_vt = first_vt + (lane >> 3);
-      const int64_t row = wrow0 + ((lane >> 2) & 1) * 32;
-      const int64_t cls = static_cast<int64_t>(my_vt) * kFwdTile + wv * (16 * kF16WV) + (lane & 3) * 32;
+      const int my_vt = first_vt + (ln >> 3);
+      const int64_t row = wrow0 + ((ln >> 2) & 1) * 32;
+      const int64_t cls = static_cast<int64_t>(my_vt) * kFwdTile + wv * (16 * kF16WV) + (ln & 3) * 32;
       if (my_vt <= vt && row < p.b && cls < p.v) {
         float mine = stat;
         if (fixed_ref) {  // the maximum was taken over raw logits
@@ -522,6 +554,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
   // the loads issued under the last tile (its own first stages once more) must land before the ring is reused
   wait_vmcnt<0>();
   __syncthreads();
+  if (WANT_LA && vt_end > vt_begin) flush_colsum(static_cast<int64_t>(vt_end - 1) * kFwdTile, (vt_end - 1) & 1);
 
   // ---- merge the four lane groups, then the two wave rows, and emit one partial per row -------
   float2* stage = reinterpret_cast<float2*>(smem);  // [NWT][WT][16]
@@ -589,7 +622,7 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   using Fast = DmaLogitTile<T, kFwdWV, kFwdWT, kFwdNWV, kFwdNWT>;
   static_assert(Fast::LDS_BYTES <= Tile::LDS_BYTES, "one LDS size serves both main loops");
   const int lds = Tile::LDS_BYTES + kFwdBiasBytes;
-  const int lds16 = lds + kF16WT * kFwdThreads * static_cast<int>(sizeof(float2));  // + the running (max, sum) pairs
+  const int lds16 = lds + kF16RunBytes;  // + the running (max, sum) pairs
   // the 16 x 16 x 32 kernel addresses token rows by 32-bit byte offsets from e and class rows by offsets from the
   // first class of a tile; shapes beyond that, and a D of one stage, take the 32 x 32 x 16 kernel
   const bool fast = aligned && (p.d % kDmaBK == 0);
@@ -610,9 +643,10 @@ static int launch_lse_forward(LseFwdParams& p, bool aligned, bool want_la, hipSt
   do {                                                                                            \
     auto kern = lse_forward16_kernel<T, GE, LA>;                                                  \
     static LdsLimitOnce lds_limit;                                                            \
-    err = lds_limit.set(kern, lds16);                                        \
+    const int bytes = lds16 + ((LA) ? kF16ColsumBytes : 0);                                       \
+    err = lds_limit.set(kern, bytes);                                                             \
     if (err != hipSuccess) return status_from_hip(err);                                           \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds16, stream, p);                    \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), bytes, stream, p);                    \
   } while (0)
   if (fast16) {
     if (want_la) CCE_LAUNCH_FWD16(true, true);
@@ -681,6 +715,7 @@ static int lse_forward_impl(const void* e, const void* c, const void* bias, cons
   p.nitems = p.nrb * p.nsplit;
   p.items_per_xcd = (p.nitems + 7) / 8;
   p.stat_cols = static_cast<int>((v + CCE_STAT_COLS - 1) / CCE_STAT_COLS);
+  p.avg_scale = kLn2 / static_cast<float>(b);
   p.sc = make_softcap(softcap);
 
   const bool aligned = aligned16(e) && aligned16(c) && (d % 8 == 0) && (stride_e % 8 == 0) &&

@@ -107,6 +107,46 @@ def test_lse_forward_spans_of_many_tiles(softcap, has_bias, shape):
     assert ((got - want).abs() <= 0.05).all()
 
 
+@pytest.mark.parametrize("softcap", [None, 20.0, 50.0])
+@pytest.mark.parametrize("shape,gathered", [((8192, 20011, 128), False), ((1000, 5000, 192), True), ((700, 2304, 256), True)])
+def test_lse_forward_column_average_over_spans(softcap, shape, gathered):
+    """logit_avg (reference cce_lse_forward.py:95-97: the mean over the rows of the soft-capped logits with bias) on
+    the 16x16x32 kernel: a workgroup sums a tile's columns in LDS and hands them over while it works on the next tile,
+    so spans of one, several and many tiles, a last tile that is cut by V, a last row block that is cut by B and rows
+    gathered through `valids` are all different code.  Two calls in a row: the entry clears the average itself."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    N, V, D = shape
+    e, c, _, bias = make_inputs(N, V, D, torch.bfloat16, seed=5, bias=True)
+    ed, cd, bd = e.to(dev), c.to(dev), bias.to(dev)
+    if gathered:
+        g = torch.Generator().manual_seed(6)
+        valids = torch.randperm(N, generator=g)[: N - 37].sort().values.to(torch.int32).to(dev)
+    else:
+        valids = None
+    B = N if valids is None else valids.numel()
+    rows = ed if valids is None else ed[valids.long()]
+    logits = rows.float() @ cd.float().T + bd.float()
+    if softcap is not None:
+        logits = torch.tanh(logits / softcap) * softcap
+    want_avg = logits.double().mean(0)
+    want_lse = torch.logsumexp(logits.double(), dim=1)
+    lse = torch.full((B,), float("nan"), dtype=torch.float32, device=dev)
+    la = torch.full((V,), float("nan"), dtype=torch.float32, device=dev)
+    ws_bytes = lib.cce_lse_forward_workspace_bytes(B, V, D)
+    ws = torch.empty((ws_bytes // 8 + 1,), dtype=torch.int64, device=dev)
+    for _ in range(2):
+        st = lib.cce_lse_forward(
+            ed.data_ptr(), cd.data_ptr(), bd.data_ptr(), valids.data_ptr() if valids is not None else None,
+            lse.data_ptr(), la.data_ptr(), None, ws.data_ptr(), ws.numel() * 8,
+            N, B, V, D, ed.stride(0), cd.stride(0), cd.stride(1),
+            softcap or 0.0, 0, torch.cuda.current_stream().cuda_stream)
+        assert st == 0, lib.cce_error_string(st)
+        torch.cuda.synchronize()
+        assert torch.allclose(lse.double(), want_lse, atol=2e-4, rtol=2e-5)
+        assert torch.allclose(la.double(), want_avg, atol=2e-4, rtol=1e-4)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("softcap", [None, 20.0])
 @pytest.mark.parametrize("has_bias", [False, True])
