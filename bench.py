@@ -204,6 +204,37 @@ def gemm_yardstick(args, w, e2, c):
     }))
 
 
+def forward_launcher(args, w, e2, c):
+    """The forward launcher alone (the reference's cce_lse_forward_kernel API), without and with the optional
+    average of the logits over the rows, timed with device events."""
+    import torch
+
+    from cut_cross_entropy.cce_lse_forward import cce_lse_forward_kernel
+
+    n, d = e2.shape
+    v = c.shape[0]
+    out = {}
+    for name, want in (("lse", False), ("lse_and_logit_avg", True)):
+        for _ in range(args.warmup):
+            cce_lse_forward_kernel(e2, c, softcap=w["softcap"], return_logit_avg=want)
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(args.steps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            cce_lse_forward_kernel(e2, c, softcap=w["softcap"], return_logit_avg=want)
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+        out[name] = {"ms_per_call": ms, "tflops": 2.0 * n * v * d / (ms * 1e-3) / 1e12}
+    print(json.dumps({
+        "metric": "forward launcher alone: lse, and lse with logit_avg (not the loss path)",
+        "config": {"workload": f"{w['name']}: E[{n},{d}] x C[{v},{d}] {args.dtype}, softcap={w['softcap']}, all rows valid"},
+        "steps": args.steps, "warmup": args.warmup, **out,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -225,6 +256,9 @@ def main():
     ap.add_argument("--gemm-yardstick", action="store_true",
                     help="instead of the loss path, time the library's plain matrix product E . C^T of the workload's "
                          "shape and input type (the logits the forward kernel never writes), and print its TFLOP/s")
+    ap.add_argument("--forward-launcher", action="store_true",
+                    help="instead of the loss path, time the forward launcher alone on the workload's shape, without "
+                         "and with its optional logit_avg output")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256)
     ap.add_argument("--traffic-probe", action="store_true",
@@ -270,6 +304,9 @@ def main():
     t = w["t"].to(dev)
     if args.gemm_yardstick:
         gemm_yardstick(args, w, e.detach().reshape(-1, w["D"]), c.detach())
+        return
+    if args.forward_launcher:
+        forward_launcher(args, w, e.detach().reshape(-1, w["D"]), c.detach())
         return
     bias = None
     if args.bias:
