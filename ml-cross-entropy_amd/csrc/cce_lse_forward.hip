@@ -32,6 +32,7 @@ struct LseFwdParams {
   int stat_cols;
   Softcap sc;
   float avg_scale;  // ln 2 / b: turns a column sum in log2 units into its share of logit_avg
+  float cap_inv;    // 1 / (-2 cap log2(e)) (soft-capping on), for the fixed-reference epilogue
 };
 
 // 8 waves (two per SIMD, so that one wave's LDS and global traffic issues in the shadow of the
@@ -309,7 +310,7 @@ static_assert(16 * kF16WV * kFwdNWV == kFwdTile && 16 * kF16WT * kFwdNWT == kFwd
 // taken on the raw logits (soft-capping is monotone) and soft-capped once per cell.  The running pair then holds
 // (cap log2(e), sum) and merges with the other spans' pairs like any other.
 template <bool GENERAL, bool CAP, bool FIXED, bool WANT_S2>
-__device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+__device__ __forceinline__ void row_block_impl(const Softcap& sc, float cap_inv, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
                                                const float* addend, int kq, float2& run, float (&bm)[kF16WV / 2],
                                                float (&s2)[kF16WV][4]) {
   float y[kF16WV][4];
@@ -328,12 +329,13 @@ __device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&
         x = dead ? 0.0f : x + add;
       }
       if (FIXED) {
+        // z = -2 cap log2(e) / (1 + t) in one fma and one reciprocal: (1 + t) / k = t / k + 1 / k
         const float t = __builtin_amdgcn_exp2f(x * sc.in_scale);
-        const float w = __builtin_amdgcn_rcpf(1.0f + t);
-        const float term = __builtin_amdgcn_exp2f(w * (-2.0f * sc.out_scale));
+        const float z = __builtin_amdgcn_rcpf(fmaf(t, cap_inv, cap_inv));
+        const float term = __builtin_amdgcn_exp2f(z);
         part += dead ? 0.0f : term;
         gm = fmaxf(gm, dead ? -INFINITY : x);
-        if (WANT_S2) s2[vi][r] = dead ? -INFINITY : fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
+        if (WANT_S2) s2[vi][r] = dead ? -INFINITY : z + sc.out_scale;
       } else {
         float v;
         if (CAP) {
@@ -342,14 +344,15 @@ __device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&
           const float w = __builtin_amdgcn_rcpf(1.0f + t);
           v = fmaf(w, -2.0f * sc.out_scale, sc.out_scale);
         } else {
-          v = x * kLog2e;
+          v = x;  // the raw logit: the maximum is scaled once per block, the exponent below in its fma
         }
         v = dead ? -INFINITY : v;
         y[vi][r] = v;
-        if (WANT_S2) s2[vi][r] = v;
+        if (WANT_S2) s2[vi][r] = CAP ? v : v * kLog2e;
         gm = fmaxf(gm, v);
       }
     }
+    if (!FIXED && !CAP) gm *= kLog2e;
     bm[vi / 2] = fmaxf(bm[vi / 2], gm);
     tm = fmaxf(tm, gm);
   }
@@ -362,7 +365,7 @@ __device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&
 #pragma unroll
     for (int vi = 0; vi < kF16WV; ++vi)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(y[vi][r] - ms);
+      for (int r = 0; r < 4; ++r) part += __builtin_amdgcn_exp2f(CAP ? y[vi][r] - ms : fmaf(y[vi][r], kLog2e, -ms));
     run.y = run.y * __builtin_amdgcn_exp2f(run.x - ms) + part;
     run.x = mn;
   }
@@ -370,12 +373,13 @@ __device__ __forceinline__ void row_block_impl(const Softcap& sc, const f32x4 (&
 
 // One uniform branch per row block: each arm is straight-line code over all 32 values.
 template <bool GENERAL, bool WANT_S2>
-__device__ __forceinline__ void row_block(const Softcap& sc, bool fixed_ref, const f32x4 (&acc)[kF16WV][kF16WT], int ti,
+__device__ __forceinline__ void row_block(const Softcap& sc, float cap_inv, bool fixed_ref,
+                                          const f32x4 (&acc)[kF16WV][kF16WT], int ti,
                                           const float* addend, int kq, float2& run, float (&bm)[kF16WV / 2],
                                           float (&s2)[kF16WV][4]) {
-  if (fixed_ref) row_block_impl<GENERAL, true, true, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
-  else if (sc.on) row_block_impl<GENERAL, true, false, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
-  else row_block_impl<GENERAL, false, false, WANT_S2>(sc, acc, ti, addend, kq, run, bm, s2);
+  if (fixed_ref) row_block_impl<GENERAL, true, true, WANT_S2>(sc, cap_inv, acc, ti, addend, kq, run, bm, s2);
+  else if (sc.on) row_block_impl<GENERAL, true, false, WANT_S2>(sc, cap_inv, acc, ti, addend, kq, run, bm, s2);
+  else row_block_impl<GENERAL, false, false, WANT_S2>(sc, cap_inv, acc, ti, addend, kq, run, bm, s2);
 }
 
 template <typename T, bool GENERAL, bool WANT_LA>
@@ -497,7 +501,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
         __builtin_amdgcn_sched_barrier(0);  // keep each row block's register use to itself
         float s2[kF16WV][4];
         float2 run = s_run[ti * kFwdThreads];
-        row_block<GENERAL, WANT_LA>(p.sc, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
+        row_block<GENERAL, WANT_LA>(p.sc, p.cap_inv, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
         s_run[ti * kFwdThreads] = run;
         if (WANT_LA) {
           const bool ok = wrow0 + ti * 16 + r16 < p.b;
@@ -717,6 +721,7 @@ static int lse_forward_impl(const void* e, const void* c, const void* bias, cons
   p.stat_cols = static_cast<int>((v + CCE_STAT_COLS - 1) / CCE_STAT_COLS);
   p.avg_scale = kLn2 / static_cast<float>(b);
   p.sc = make_softcap(softcap);
+  p.cap_inv = p.sc.on ? 1.0f / (-2.0f * p.sc.out_scale) : 0.0f;
 
   const bool aligned = aligned16(e) && aligned16(c) && (d % 8 == 0) && (stride_e % 8 == 0) &&
                        (stride_cv % 8 == 0) && (stride_cd == 1);
