@@ -482,6 +482,9 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
     // ---- epilogue: (bias, mask,) soft-cap, online max / sum-exp ---------------------------------
     const int64_t vw0 = v0 + wv * (16 * kF16WV);  // first class of this wave
     const float* wave_addend = addend + wv * (16 * kF16WV);
+    // A tile with no bias and no class past the end of the vocabulary has nothing to add and nothing to mask: of a
+    // vocabulary that is no multiple of 256 only the last tile pays for the per-class addend.
+    const bool plain_tile = GENERAL && p.bias == nullptr && v0 + kFwdTile <= p.v;
     float la[WANT_LA ? kF16WV : 1][4];  // this lane's sums over its four rows of the tile, log2 units
     if (WANT_LA) {
       if (vt > vt_begin) flush_colsum(v0 - kFwdTile, (vt - 1) & 1);
@@ -501,7 +504,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
         __builtin_amdgcn_sched_barrier(0);  // keep each row block's register use to itself
         float s2[kF16WV][4];
         float2 run = s_run[ti * kFwdThreads];
-        row_block<GENERAL, WANT_LA>(p.sc, p.cap_inv, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
+        if (GENERAL && plain_tile) row_block<false, WANT_LA>(p.sc, p.cap_inv, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
+        else row_block<GENERAL, WANT_LA>(p.sc, p.cap_inv, fixed_ref, acc, ti, wave_addend, kq, run, bm, s2);
         s_run[ti * kFwdThreads] = run;
         if (WANT_LA) {
           const bool ok = wrow0 + ti * 16 + r16 < p.b;
