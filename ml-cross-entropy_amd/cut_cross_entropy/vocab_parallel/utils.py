@@ -11,8 +11,6 @@ returning shard-local values.
 from dataclasses import dataclass
 from typing import Any, Optional, Tuple
 
-import torch
-
 
 def partition_n_into_range(n: int, rank: int, world_size: int) -> Tuple[int, int]:
     """Contiguous split of range(n): every rank gets n // world_size items and the

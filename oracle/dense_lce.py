@@ -32,11 +32,9 @@ No function here is "parity unpinned".
 
 from __future__ import annotations
 
-import math
 from typing import Optional, Tuple
 
 import torch
-import torch.nn.functional as F
 
 IGNORE_INDEX = -100  # cut_cross_entropy/constants.py:2
 

@@ -1,7 +1,6 @@
 """The C-ABI library loads and exports every symbol include/cce_hip.h declares; the host-only
 queries answer without a GPU.  No compute entry point is called here."""
 
-import ctypes
 import os
 import re
 

@@ -2,8 +2,6 @@
 full size for the headline shape), plus the properties that only show at scale: gradient
 filtering with the no-recompute shortcut, determinism, class permutation, vocabulary shards."""
 
-import math
-
 import pytest
 import torch
 

@@ -1,7 +1,5 @@
 """Parity of the three HIP kernels, called through the C ABI, against the CPU oracle."""
 
-import ctypes
-
 import pytest
 import torch
 

@@ -2,8 +2,6 @@
 answer of the reference's own tests, a library routine, brute force, or a mathematical identity
 chosen so that a dropped term, a wrong sign or a wrong index fails."""
 
-import itertools
-
 import numpy as np
 import pytest
 import scipy.special
