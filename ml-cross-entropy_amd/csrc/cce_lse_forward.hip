@@ -480,7 +480,6 @@ __global__ __launch_bounds__(kFwdThreads, 1) void lse_forward16_kernel(LseFwdPar
     });
 
     // ---- epilogue: (bias, mask,) soft-cap, online max / sum-exp ---------------------------------
-    const int64_t vw0 = v0 + wv * (16 * kF16WV);  // first class of this wave
     const float* wave_addend = addend + wv * (16 * kF16WV);
     // A tile with no bias and no class past the end of the vocabulary has nothing to add and nothing to mask: of a
     // vocabulary that is no multiple of 256 only the last tile pays for the per-class addend.

@@ -169,7 +169,7 @@ struct Tile4 {
     const int32_t* pair = l.b_rows + (k0 + row_kmajor(q, g.wave));  // uniform
     ids.v[B_GATHER ? q : 0] = pair[g.half];
   }
-  static __device__ __forceinline__ void prep_b(Ptrs& p, int q, const Ids& ids, const Loop& l, const Geometry& g) {
+  static __device__ __forceinline__ void prep_b(Ptrs& p, int q, const Ids& ids, const Loop& l, const Geometry&) {
     if (!B_GATHER) return;
     p.b[B_GATHER ? q : 0] = l.b_lane + static_cast<uint64_t>(static_cast<uint32_t>(ids.v[B_GATHER ? q : 0])) * l.b_stride;
   }
